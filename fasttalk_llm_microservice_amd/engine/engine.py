@@ -70,14 +70,19 @@ class LLMEngine:
         self.runner = runner
         self.max_model_len = runner.max_model_len
         R = rt()
-        self.bm = R.BlockManager(runner.num_blocks, cfg.block_size, cfg.enable_prefix_caching)
+        # recurrent state cannot be rebuilt from cached KV blocks: a sequence of a model
+        # with state slots always computes its own prefix
+        state_slots = int(getattr(runner, "num_state_slots", 0))
+        self.bm = R.BlockManager(runner.num_blocks, cfg.block_size,
+                                 cfg.enable_prefix_caching and not state_slots)
         self.detok = R.Detokenizer(self.tokenizer.id_to_bytes)
         self.scheduler = Scheduler(self.bm, cfg.block_size, cfg.max_num_seqs,
                                    cfg.max_num_batched_tokens, self.max_model_len,
                                    host_blocks=getattr(runner, "num_host_blocks", 0),
                                    prefill_chunk=cfg.prefill_chunk,
                                    chunk_counts_decode=cfg.prefill_chunk_rows,
-                                   guided_prefill_cap=cfg.guided_prefill_cap)
+                                   guided_prefill_cap=cfg.guided_prefill_cap,
+                                   state_slots=state_slots)
         self.stop_ids = set(self.tokenizer.stop_ids) | set(self.model_cfg.eos_token_ids)
         self._trie = None
         # jump-forward over grammar-forced runs (ENGINE_JUMP_FORWARD=0 disables)
@@ -802,6 +807,52 @@ class LLMEngine:
         if emit and seq.on_output is not None:
             seq.on_output(out)
         return out
+
+    # ------------------------------------------------------------------ given steps
+    def replay_step(self, entries, end=()) -> np.ndarray:
+        """One step whose rows the caller dictates (replaying a recorded schedule,
+        scoring): ``entries`` = [(request id, next token ids, wanted offsets)], all run
+        as one batch through the scheduler's block / state-slot pools and the runner's
+        step function.  A request is admitted at its first entry; ``end`` lists the
+        requests that are finished after this step (their blocks and slot go back).
+        Returns the logits at the wanted offsets, fp32 [wanted, vocab], in the order of
+        the entries."""
+        if self._inflight:
+            raise EngineError("replay_step with queued steps")
+        sched = self.scheduler
+        items = []
+        for rid, toks, _ in entries:
+            seq = sched.by_id.get(rid)
+            if seq is None:
+                seq = Sequence(rid, list(toks), SamplingParams(temperature=0.0, max_tokens=1 << 30))
+                sched.admit_given(seq)
+            else:
+                for t in toks:
+                    seq.append(int(t))
+            if seq.n_tokens > self.max_model_len:
+                raise EngineError(f"request {rid}: {seq.n_tokens} tokens exceed max_model_len")
+            items.append((seq, len(toks)))
+        logits = np.zeros((0, self.model_cfg.vocab_size), np.float32)
+        if items:
+            batch = sched.schedule_given(items)
+            # row bases in the step's order: decode rows, then the prefill chunks
+            base, r = {}, len(batch.decode_seqs)
+            for i, s in enumerate(batch.decode_seqs):
+                base[s.request_id] = i
+            for s, n in zip(batch.prefill_seqs, batch.prefill_tokens):
+                base[s.request_id] = r
+                r += n
+            batch.logit_rows = [base[rid] + int(w) for rid, _, want in entries for w in want]
+            self._executing = batch
+            logits = self.runner.execute(batch, None, logits_only=True)
+            self._executing = None
+            sched.post_step(batch)
+            self.stats["given_steps"] += 1
+        for rid in end:
+            seq = sched.by_id.get(rid)
+            if seq is not None:
+                sched.finish(seq, "stop")
+        return logits
 
     # ------------------------------------------------------------------ convenience
     def generate(self, prompts: List[List[int]], params: SamplingParams) -> List[List[int]]:

@@ -21,7 +21,8 @@ import torch
 
 from .. import ops
 from ..models.config import ModelConfig
-from ..models.llama import AttnMeta, LlamaModel
+from ..models.llama import AttnMeta
+from ..models.registry import build_model
 from ..parallel.comm import SINGLE, TPComm
 from .config import EngineConfig
 from .scheduler import ScheduledBatch
@@ -201,8 +202,13 @@ class ModelRunner:
         self.max_blocks_per_seq = (self.max_model_len + self.bs - 1) // self.bs
 
         t0 = time.time()
-        self.model = LlamaModel(model_cfg, self.device, self.dtype, comm, self.max_model_len,
-                                quantization=cfg.quantization)
+        # the architecture registry picks the model class (models/registry.py)
+        self.model = build_model(model_cfg, self.device, self.dtype, comm, self.max_model_len,
+                                 quantization=cfg.quantization)
+        # models whose mixers keep per-sequence recurrent state / take varlen row
+        # segments (ops.mixers.Segments) instead of the Llama attention plans
+        self.stateful = bool(getattr(self.model, "needs_state_slots", False))
+        self.num_state_slots = cfg.max_num_seqs if self.stateful else 0
         if cfg.weights and cfg.weights != "random":
             self.model.load_checkpoint(cfg.weights)
         else:
@@ -215,11 +221,17 @@ class ModelRunner:
         # budget plus a decode row per sequence
         self.invariant = bool(getattr(cfg, "batch_invariant", False))
         if self.invariant:
+            if self.stateful:
+                raise ValueError("batch_invariant is a mode of the Llama kernel plans")
             self.model.set_batch_invariant(max(cfg.max_num_batched_tokens, cfg.max_num_seqs)
                                            + cfg.max_num_seqs)
         self.kv_dtype = cfg.kv_torch_dtype(self.dtype)
         self.num_blocks = self._decide_num_blocks()
-        self.kv = self.model.allocate_kv_cache(self.num_blocks, self.bs, self.kv_dtype)
+        if self.stateful:
+            self.kv = self.model.allocate_kv_cache(self.num_blocks, self.bs, self.kv_dtype,
+                                                   num_slots=self.num_state_slots)
+        else:
+            self.kv = self.model.allocate_kv_cache(self.num_blocks, self.bs, self.kv_dtype)
         # FT_KERNEL_CHECKS=1: the bounds-checked kernel build validates every index it
         # is handed against the tensors of the launch (this pool's blocks, the rotary
         # table's rows, the vocab) and reports into this word, read after each step
@@ -232,15 +244,22 @@ class ModelRunner:
                         self.model.cos_sin.shape[0], self.mcfg.vocab_size)
         # E6 host swap pool (--swap-space): capped at 2x the device pool, allocated
         # (pinned) on the first swap-out so an idle server does not pin host memory
-        k0 = self.kv[0][0]
-        self.kv_block_elems = k0.numel() // k0.shape[0]
-        host_block_bytes = 2 * len(self.kv) * self.kv_block_elems * k0.element_size()
-        self.num_host_blocks = min(int(cfg.swap_space_gb * (1 << 30)) // host_block_bytes,
-                                   2 * self.num_blocks)
+        if self.stateful:
+            # a preempted sequence is recomputed: its recurrent state has no host copy
+            self.kv_block_elems = 0
+            self.num_host_blocks = 0
+        else:
+            k0 = self.kv[0][0]
+            self.kv_block_elems = k0.numel() // k0.shape[0]
+            host_block_bytes = 2 * len(self.kv) * self.kv_block_elems * k0.element_size()
+            self.num_host_blocks = min(int(cfg.swap_space_gb * (1 << 30)) // host_block_bytes,
+                                       2 * self.num_blocks)
         self.host_kv = None
         self.swap_staging = None
         self.kv_ptrs = None
-        nq, d = self.model.nq, self.model.d
+        # (query heads, kv heads, head dim) of the Llama attention kernels' work plans
+        nq, nkv, d = (1, 1, 64) if self.stateful else (self.model.nq, self.model.nkv, self.model.d)
+        self.attn_dims = None if self.stateful else (nq, nkv, d)
 
         # -------- static decode buffers (graph inputs) --------
         self.graph_sizes = sorted(b for b in cfg.graph_batch_sizes if b <= cfg.max_num_seqs) or [1]
@@ -298,10 +317,10 @@ class ModelRunner:
         # decode-attention partials: one slot per (sequence, kv head) + one per wave
         # of the kernel's grid (any step has at most max_num_seqs decode rows)
         self.max_decode_rows = max(mb, cfg.max_num_seqs)
-        n_out, n_ml = ops.decode_workspace(self.max_decode_rows, nq, self.model.nkv, d,
-                                           waves=None if self.is_gpu else 0,
-                                           piece=ops.DECODE_INV_PIECE if self.invariant else 0,
-                                           max_len=self.max_blocks_per_seq * self.bs)
+        n_out, n_ml = (0, 0) if self.stateful else ops.decode_workspace(
+            self.max_decode_rows, nq, nkv, d, waves=None if self.is_gpu else 0,
+            piece=ops.DECODE_INV_PIECE if self.invariant else 0,
+            max_len=self.max_blocks_per_seq * self.bs)
         self.tmp_out = torch.empty(max(1, n_out), dtype=torch.float32, device=dv)
         self.tmp_ml = torch.empty(max(1, n_ml), dtype=torch.float32, device=dv)
         # split-KV prefill partials (ops.build_prefill_tiles): 128 slots = 128 MiB fp32
@@ -314,24 +333,25 @@ class ModelRunner:
         self.pf_max_partials = ops.PREFILL_MAX_PARTIALS
         if self.invariant:
             pieces = -(-self.max_model_len // (ops.PREFILL_BK * ops.PREFILL_INV_CHUNK))
-            qblocks = -(-cfg.max_num_batched_tokens // ops.prefill_tile_tokens(nq, self.model.nkv))
+            qblocks = -(-cfg.max_num_batched_tokens // ops.prefill_tile_tokens(nq, nkv))
             self.pf_max_partials = max(ops.PREFILL_MAX_PARTIALS,
                                        (qblocks + cfg.max_num_seqs) * pieces)
-        if self.is_gpu and (self.invariant or os.environ.get("FT_PREFILL_SPLIT", "1") == "1"):
-            n_po, n_pml = ops.prefill_partials(self.model.nkv, d, self.pf_max_partials)
+        if self.is_gpu and not self.stateful and \
+                (self.invariant or os.environ.get("FT_PREFILL_SPLIT", "1") == "1"):
+            n_po, n_pml = ops.prefill_partials(nkv, d, self.pf_max_partials)
             self.pf_part_o = torch.empty(n_po, dtype=torch.float32, device=dv)
             self.pf_part_ml = torch.empty(n_pml, dtype=torch.float32, device=dv)
         # in-launch combine tickets (FT_DECODE_FUSED_COMBINE=0: separate combine kernel):
         # with the kernel at one workgroup per CU the last-arriver merge matches or beats
         # the combine kernel and saves a launch per layer (csrc/kernels/attn_decode.hip)
-        self.dec_counters = ops.decode_counters(self.max_decode_rows, self.model.nkv, dv) \
-            if self.is_gpu and (self.invariant or os.environ.get("FT_DECODE_FUSED_COMBINE", "1") == "1") \
-            else None
+        self.dec_counters = ops.decode_counters(self.max_decode_rows, nkv, dv) \
+            if self.is_gpu and not self.stateful and \
+            (self.invariant or os.environ.get("FT_DECODE_FUSED_COMBINE", "1") == "1") else None
         self._done_event = torch.cuda.Event() if self.is_gpu else None
         # persistent decode block: its sticky give-up word (ctl[2]) is copied to pinned
         # memory every BLOCK_CHECK_EVERY waits and read at the next check (never a sync)
         self._blk_host = torch.zeros(1, dtype=torch.int32, pin_memory=True) \
-            if self.is_gpu and self.model.block else None
+            if self.is_gpu and getattr(self.model, "block", False) else None
         self._blk_event = torch.cuda.Event() if self._blk_host is not None else None
         self._blk_armed = False
         self._blk_waits = 0
@@ -345,7 +365,8 @@ class ModelRunner:
         # ENGINE_GUIDED_PIPELINE=0: guided batches run one synchronous step at a time
         self.guided_pipeline = os.environ.get("ENGINE_GUIDED_PIPELINE", "1") != "0"
         self.graph_pool = None
-        self.use_graphs = self.is_gpu and not cfg.enforce_eager and comm.graph_safe()
+        self.use_graphs = self.is_gpu and not cfg.enforce_eager and comm.graph_safe() \
+            and getattr(self.model, "supports_graphs", True)
         # FT_FAULT_TP_STALL="<n>:<seconds>" (TP workers): before executing the n-th
         # decode graph message, stall until rank 0's custom all-reduce has run out of
         # spin budget (its error word is set; at most <seconds>) -- the fault test
@@ -426,8 +447,11 @@ class ModelRunner:
 
     def _decide_num_blocks(self) -> int:
         cfg = self.cfg
-        per_block = self.mcfg.num_layers * 2 * self.model.nkv * self.model.d * self.bs * \
-            torch.tensor([], dtype=self.kv_dtype).element_size()
+        if hasattr(self.model, "kv_block_bytes"):
+            per_block = self.model.kv_block_bytes(self.bs, self.kv_dtype)
+        else:
+            per_block = self.mcfg.num_layers * 2 * self.model.nkv * self.model.d * self.bs * \
+                torch.tensor([], dtype=self.kv_dtype).element_size()
         if cfg.num_kv_blocks:
             n = cfg.num_kv_blocks
         elif self.is_gpu:
@@ -457,12 +481,21 @@ class ModelRunner:
 
     # ------------------------------------------------------------------ execution
     @torch.inference_mode()
-    def execute(self, batch: ScheduledBatch, masks: Optional[np.ndarray] = None) -> List[int]:
+    def execute(self, batch: ScheduledBatch, masks: Optional[np.ndarray] = None,
+                logits_only: bool = False):
         """Runs one step; returns sampled ids for ``batch.sampled_seqs()`` in order.
 
         Decode-only steps replay a hipGraph; steps that carry prefill chunks run
-        eagerly as one mixed forward pass (decode rows first)."""
+        eagerly as one mixed forward pass (decode rows first).  ``logits_only``: nothing
+        is sampled; the step's logits rows (``batch.logit_rows``, or the rows that would
+        be sampled) come back as an fp32 host array [rows, vocab]."""
         self._assert_no_pending_split("execute")
+        if logits_only:
+            if self.bcast is not None:
+                raise RuntimeError("logits_only steps run in a single process")
+            host = self._mixed_host(batch)
+            host["logits_only"] = True
+            return self._mixed_run(host, None)
         if batch.has_prefill:
             if self._gaps is not None:
                 self._gap_mark(True, "m")   # closed by _wait, right after the last launch
@@ -541,13 +574,34 @@ class ModelRunner:
             slots.append(blk[p // bs] * bs + p % bs)
             seq_lens[i] = a + n
             qsl[i + 1] = qsl[i] + n
-        tiles, combine = ops.build_prefill_tiles(
-            ntoks, ops.prefill_tile_tokens(self.model.nq, self.model.nkv),
-            seq_lens=seq_lens if self.pf_part_o is not None else None, nkv=self.model.nkv,
-            num_cus=self.num_cus, max_partials=self.pf_max_partials,
-            fixed_chunk=ops.PREFILL_INV_CHUNK if self.invariant else 0)
+        if self.stateful:
+            tiles, combine = [], []
+            # one segment per scheduled sequence, decode rows first (ops.mixers.Segments)
+            ns = nd + len(pseqs)
+            sg_bt = np.zeros((max(1, ns), max([len(s.block_ids) for s in dseqs + pseqs] or [1])),
+                             np.int32)
+            for i, s in enumerate(dseqs + pseqs):
+                sg_bt[i, : len(s.block_ids)] = s.block_ids
+            d_pos0 = pos[0] if nd else np.zeros(0, np.int32)
+            p_pos0 = np.asarray([seq_lens[i] - ntoks[i] for i in range(len(pseqs))], np.int32)
+            host.update(
+                sg_start=np.concatenate([np.arange(nd, dtype=np.int32), nd + qsl]).astype(np.int32),
+                sg_pos0=np.concatenate([d_pos0, p_pos0]).astype(np.int32),
+                sg_slot=np.asarray([s.state_slot for s in dseqs + pseqs] or [0], np.int32),
+                sg_len=np.concatenate([d_pos0 + 1, seq_lens]).astype(np.int32) if ns
+                else np.zeros(1, np.int32),
+                sg_bt=sg_bt, num_segs=ns, max_rows=max([1] * bool(nd) + ntoks + [0]),
+                max_kv=int(max([0] + [int(x) for x in d_pos0 + 1] + [int(x) for x in seq_lens])))
+        else:
+            tiles, combine = ops.build_prefill_tiles(
+                ntoks, ops.prefill_tile_tokens(self.attn_dims[0], self.attn_dims[1]),
+                seq_lens=seq_lens if self.pf_part_o is not None else None, nkv=self.attn_dims[1],
+                num_cus=self.num_cus, max_partials=self.pf_max_partials,
+                fixed_chunk=ops.PREFILL_INV_CHUNK if self.invariant else 0)
         # logits rows: every decode row + the last row of each prompt that completes
         lrows = list(range(nd)) + [nd + int(qsl[i + 1]) - 1 for i, sm in enumerate(psamp) if sm]
+        if batch.logit_rows is not None:
+            lrows = list(batch.logit_rows)
         host.update(ids=np.concatenate(ids).astype(np.int32), pos=np.concatenate(pos).astype(np.int32),
                     slots=np.concatenate(slots).astype(np.int32), lrows=np.asarray(lrows, np.int64),
                     bt=bt, seq_lens=seq_lens, qsl=qsl, tiles=np.asarray(tiles, np.int32).reshape(-1),
@@ -555,7 +609,7 @@ class ModelRunner:
                     num_combine=len(combine),
                     num_partials=sum(c[3] for c in combine))
         sseqs = dseqs + [s for s, sm in zip(pseqs, psamp) if sm]
-        host["sampling"] = self._sampling_arrays(sseqs)
+        host["sampling"] = self._sampling_arrays(sseqs if batch.logit_rows is None else [])
         if self.logits_tap_ids is not None:
             self._tap_rows = [s.request_id for s in sseqs]
         return host
@@ -585,9 +639,12 @@ class ModelRunner:
             if nd > self.max_decode_rows:
                 raise ValueError(f"{nd} decode rows exceed max_num_seqs {self.max_decode_rows}")
             names += ["d_bt", "d_sl"]
+        if self.stateful:
+            names += self._SEG_NAMES
         arrays = [host[k] for k in names]
         has_logits = len(host["lrows"]) > 0
-        if has_logits:
+        logits_only = bool(host.get("logits_only"))
+        if has_logits and not logits_only:
             arrays += list(host["sampling"])
             if masks is not None:
                 arrays.append(masks)
@@ -601,6 +658,8 @@ class ModelRunner:
             block_tables=d["bt"], seq_lens=d["seq_lens"],
             q_start_loc=d["qsl"] if self.is_gpu else torch.from_numpy(qsl),
             tile_info=d["tiles"], num_tiles=host["num_tiles"])
+        if self.stateful:
+            meta.segments = self._segments(d, host)
         if host.get("num_combine", 0):
             meta.pf_part_o, meta.pf_part_ml = self.pf_part_o, self.pf_part_ml
             meta.pf_combine, meta.pf_num_combine = d["combine"], host["num_combine"]
@@ -611,6 +670,17 @@ class ModelRunner:
             meta.tmp_out, meta.tmp_ml = self.tmp_out, self.tmp_ml
             meta.dec_counters = self.dec_counters
         h = self.model.forward(d["ids"], meta, self.kv)
+        if logits_only:
+            if not has_logits:
+                self._wait() if self.is_gpu else None
+                return np.zeros((0, self.mcfg.vocab_size), np.float32)
+            logits = self.model.compute_logits(h).float()
+            if not self.is_gpu:
+                return logits.numpy()
+            out = torch.empty(logits.shape, dtype=torch.float32, pin_memory=True)
+            out.copy_(logits, non_blocking=True)
+            self._wait()
+            return out.numpy()
         if not has_logits:
             # a middle chunk of a chunked prefill samples nothing, but its all-reduces
             # wrote KV blocks that post_step commits to the prefix cache: check the
@@ -626,6 +696,16 @@ class ModelRunner:
         samp = dev[k:k + 5]
         dmask = dev[k + 5] if masks is not None else None
         return self._sample(h, host["sampling"], masks, dev_sampling=samp, dev_mask=dmask)
+
+    _SEG_NAMES = ["sg_start", "sg_pos0", "sg_slot", "sg_len", "sg_bt"]
+
+    @staticmethod
+    def _segments(d, host):
+        from ..ops.mixers import Segments
+
+        return Segments(start=d["sg_start"], pos0=d["sg_pos0"], slot=d["sg_slot"], kv_len=d["sg_len"],
+                        block_tables=d["sg_bt"], num=host["num_segs"], max_rows=host["max_rows"],
+                        max_kv=host["max_kv"])
 
     def _wait(self, ev=None):
         """Block until the GPU work queued so far (or up to ``ev``) is done WITHOUT
@@ -910,6 +990,8 @@ class ModelRunner:
         names = ["pos", "slots", "lrows", "bt", "seq_lens", "qsl", "tiles", "ids", "combine"]
         if nd:
             names += ["d_bt", "d_sl"]
+        if self.stateful:
+            names += self._SEG_NAMES
         arrays = [host[k] for k in names] + list(host["sampling"])
         # rowmap[i] < 0: row i's sequence has no queued step (it joined after the last
         # queued step was built); its id is its last token, already in host["ids"]
@@ -938,6 +1020,8 @@ class ModelRunner:
             block_tables=d["bt"], seq_lens=d["seq_lens"],
             q_start_loc=d["qsl"] if self.is_gpu else torch.from_numpy(host["qsl"]),
             tile_info=d["tiles"], num_tiles=host["num_tiles"])
+        if self.stateful:
+            meta.segments = self._segments(d, host)
         if host.get("num_combine", 0):
             meta.pf_part_o, meta.pf_part_ml = self.pf_part_o, self.pf_part_ml
             meta.pf_combine, meta.pf_num_combine = d["combine"], host["num_combine"]

@@ -46,6 +46,10 @@ class ScheduledBatch:
     # scheduled (Scheduler.stamp); empty for batches built outside the scheduler
     prefill_start: List[int] = dataclasses.field(default_factory=list)
     prefill_epoch: List[int] = dataclasses.field(default_factory=list)
+    # rows of the step (decode rows first, then the prefill chunks in order) whose
+    # logits are wanted, in the order wanted; None: every decode row and the last row
+    # of each sampled chunk (Scheduler.schedule_given: scoring / replay)
+    logit_rows: Optional[List[int]] = None
 
     @property
     def is_prefill(self) -> bool:
@@ -87,12 +91,34 @@ class HostSwapPool:
         self._free.extend(reversed(slots))
 
 
+class StateSlotPool:
+    """Slots of the recurrent-state tensors (one slot = the state of every recurrent
+    layer run for one sequence).  A slot is handed out when a sequence's first chunk is
+    scheduled and goes back with its KV blocks; a sequence that starts at position 0
+    starts from a zero state whatever the slot held (the kernels do not read it)."""
+
+    def __init__(self, num_slots: int):
+        self.num_slots = num_slots
+        self._free = list(range(num_slots - 1, -1, -1))
+
+    def num_free(self) -> int:
+        return len(self._free)
+
+    def allocate(self) -> int:
+        return self._free.pop() if self._free else -1
+
+    def release(self, slot: int):
+        if slot >= 0:
+            self._free.append(slot)
+
+
 class Scheduler:
     def __init__(self, block_manager, block_size: int, max_num_seqs: int,
                  max_num_batched_tokens: int, max_model_len: int, host_blocks: int = 0,
                  prefill_chunk: int = 0, chunk_counts_decode: bool = False,
-                 guided_prefill_cap: int = 0):
+                 guided_prefill_cap: int = 0, state_slots: int = 0):
         self.bm = block_manager
+        self.slots = StateSlotPool(state_slots) if state_slots > 0 else None
         self.bs = block_size
         self.max_num_seqs = max_num_seqs
         self.max_tokens = max_num_batched_tokens
@@ -173,6 +199,17 @@ class Scheduler:
         if seq.host_slots:
             self.host.release(seq.host_slots)
             seq.host_slots = []
+        if self.slots is not None and seq.state_slot >= 0:
+            self.slots.release(seq.state_slot)
+            seq.state_slot = -1
+
+    def _take_slot(self, seq: Sequence) -> bool:
+        """A state slot for a sequence about to run its first rows (True if it has one
+        or needs none)."""
+        if self.slots is None or seq.state_slot >= 0:
+            return True
+        seq.state_slot = self.slots.allocate()
+        return seq.state_slot >= 0
 
     def finish(self, seq: Sequence, reason: str):
         seq.status = SeqStatus.FINISHED
@@ -340,6 +377,8 @@ class Scheduler:
                 soft = 0
             limit = budget if not seqs or not soft else min(budget, soft - used)
             chunk = min(remaining, limit)
+            if not self._take_slot(seq):
+                break   # every state slot is held by a running sequence: wait for one
             need = self._blocks_needed(seq, start + chunk)
             if need and not self.bm.can_allocate(need) and self._release_background():
                 pass  # a warm-up's blocks went back to the pool first (optional work)
@@ -411,6 +450,8 @@ class Scheduler:
         remaining = seq.n_tokens - start
         chunk = min(remaining, room)
         need = self._blocks_needed(seq, start + chunk)
+        if not self._take_slot(seq):
+            return
         if need and not self.bm.can_allocate(need):
             self.background.popleft()
             self.release(seq)
@@ -473,6 +514,37 @@ class Scheduler:
                     continue
                 seq.block_ids.extend(self.bm.allocate(need))
         return list(self.running)
+
+    # ------------------------------------------------------------------ given steps
+    def admit_given(self, seq: Sequence):
+        """Registers a sequence whose steps the caller dictates (schedule_given)."""
+        self.by_id[seq.request_id] = seq
+
+    def schedule_given(self, items: List[Tuple[Sequence, int]]) -> ScheduledBatch:
+        """A step whose rows are dictated (replay of a recorded schedule, scoring):
+        for each (sequence, n) its next n tokens, which the caller has appended to it.
+        Blocks and state slots come from the same pools as in :meth:`schedule`; one
+        new token of a sequence that already has context is a decode row, anything
+        else a prefill chunk.  Nothing is sampled (``logit_rows`` says which logits
+        the caller wants)."""
+        decode, pseqs, ptok = [], [], []
+        for seq, n in items:
+            start = seq.num_computed
+            if n < 1 or start + n != seq.n_tokens:
+                raise ValueError("a given step must carry exactly the sequence's pending tokens")
+            if not self._take_slot(seq):
+                raise RuntimeError("no free state slot")
+            need = self._blocks_needed(seq, start + n)
+            if need:
+                if not self.bm.can_allocate(need):
+                    raise RuntimeError("KV pool exhausted")
+                seq.block_ids.extend(self.bm.allocate(need))
+            if n == 1 and start > 0:
+                decode.append(seq)
+            else:
+                pseqs.append(seq)
+                ptok.append(n)
+        return self.stamp(ScheduledBatch(decode, pseqs, ptok, [False] * len(pseqs)))
 
     def post_step(self, batch: ScheduledBatch):
         items = [(s, 1, False, None) for s in batch.decode_seqs] + \

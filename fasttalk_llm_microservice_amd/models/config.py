@@ -31,6 +31,7 @@ class ModelConfig:
     max_position_embeddings: int = 8192
     bos_token_id: int = 128000
     eos_token_ids: tuple = (128001, 128008, 128009)
+    architecture = "llama"     # key into models.registry.ARCHITECTURES
 
     @property
     def q_size(self) -> int:
@@ -100,28 +101,38 @@ ALIASES = {
 }
 
 
-def resolve_model(name_or_path: str) -> ModelConfig:
-    """Resolve a registry name, alias, or a HF checkpoint dir with config.json."""
+def resolve_model(name_or_path: str):
+    """Resolve a registry name, alias, or a checkpoint dir with config.json (the
+    directory's architecture decides the configuration class: models.registry)."""
+    from . import registry
+
     key = name_or_path.strip()
     if os.path.isdir(key) and os.path.exists(os.path.join(key, "config.json")):
-        return from_hf_config(os.path.join(key, "config.json"))
+        return registry.config_from_dir(key)
     low = key.lower()
     if low in MODELS:
         return MODELS[low]
     if low in ALIASES:
         return MODELS[ALIASES[low]]
+    cfg = registry.preset(low)
+    if cfg is not None:
+        return cfg
     raise KeyError(f"unknown model '{name_or_path}'; known: {sorted(MODELS)} + aliases")
 
 
 def from_hf_config(path: str) -> ModelConfig:
     with open(path) as f:
         c = json.load(f)
+    return llama_from_dict(c, os.path.basename(os.path.dirname(path)) or "hf-model")
+
+
+def llama_from_dict(c: dict, name: str) -> ModelConfig:
     h = c["hidden_size"]
     nh = c["num_attention_heads"]
     eos = c.get("eos_token_id", 128009)
     eos = tuple(eos) if isinstance(eos, list) else (eos,)
     return ModelConfig(
-        name=os.path.basename(os.path.dirname(path)) or "hf-model",
+        name=name,
         hidden_size=h,
         num_layers=c["num_hidden_layers"],
         num_heads=nh,

@@ -59,6 +59,9 @@ class AttnMeta:
     pf_combine: Optional[torch.Tensor] = None
     pf_num_combine: int = 0
     pf_num_partials: int = 0
+    # row segments of the step, one per scheduled sequence, decode rows first
+    # (ops.mixers.Segments): models with recurrent state slots / varlen mixer kernels
+    segments: Optional[object] = None
 
     @property
     def is_prefill(self) -> bool:

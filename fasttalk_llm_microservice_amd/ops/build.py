@@ -6,6 +6,10 @@ repository snapshot to a GPU box:
 * ``fasttalk_llm_microservice_amd/_C.so``  -- the gfx950 HIP kernels in
   ``csrc/kernels/*.hip`` (compiled with ``hipcc --offload-arch=gfx950``) plus the
   torch bindings ``csrc/bindings.cpp``.
+* ``fasttalk_llm_microservice_amd/_C_mixers.so`` -- the sequence-mixer / MoE kernels
+  in ``csrc/mixers/*.hip`` with their bindings ``csrc/mixers/bindings.cpp`` (fp32 and
+  bf16 instantiations).  A separate extension, so a model that only needs these
+  kernels builds these alone on a fresh checkout.
 * ``fasttalk_llm_microservice_amd/_rt.so`` -- the host runtime in
   ``csrc/runtime/*.cpp`` (KV block manager, detokenizer, JSON-schema token FSM,
   batch metadata builder), plain C++17 + pybind11, no torch / HIP dependency so
@@ -92,6 +96,11 @@ def _compile(src: Path, obj: Path, cmd: list, deps: list, force: bool) -> bool:
     return True
 
 
+# Device code is built without the packed-fp32 VALU forms (v_pk_add/mul/fma_f32): the
+# compiler then emits scalar fp32 ops for float and float2 code alike.  (A device-only
+# target feature: hipcc's host pass warns that it does not know it, which is harmless.)
+NO_PK_F32 = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
 # Per-kernel extra flags.  The attention kernels keep their MFMA accumulators in
 # VGPRs (gfx950's unified register file): in the AGPR form hipcc copied the O
 # accumulator AGPR -> VGPR -> AGPR around every online-softmax rescale (64 extra
@@ -116,11 +125,11 @@ def build_kernels(force: bool = False, jobs: int = 8, verbose: bool = True,
     extra = ["-DFT_KERNEL_CHECKS=1"] if checked else []
     bdir = BUILD / ("checked" if checked else "")
     kflags = [HIPCC, f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC",
-              f"-I{CSRC / 'include'}", "-munsafe-fp-atomics"] + extra
+              f"-I{CSRC / 'include'}", "-munsafe-fp-atomics"] + NO_PK_F32 + extra
     tflags, ldflags = _torch_flags()
     tflags = [f for f in tflags if not f.startswith("-DTORCH_EXTENSION_NAME=")] + \
         [f"-DTORCH_EXTENSION_NAME={name}"]
-    bflags = [HIPCC, f"--offload-arch={ARCH}"] + tflags + [f"-I{CSRC / 'include'}"] + extra
+    bflags = [HIPCC, f"--offload-arch={ARCH}"] + tflags + [f"-I{CSRC / 'include'}"] + NO_PK_F32 + extra
     jobs_list = [(k, bdir / "kernels" / (k.stem + ".o"), kflags + KERNEL_FLAGS.get(k.stem, []), headers)
                  for k in kernels]
     jobs_list.append((CSRC / "bindings.cpp", bdir / "bindings.o", bflags + ["-x", "hip"], headers))
@@ -138,6 +147,40 @@ def build_kernels(force: bool = False, jobs: int = 8, verbose: bool = True,
         _run([HIPCC, f"--offload-arch={ARCH}", "-shared", "-fPIC", *objs, "-o", str(out), *ldflags])
         if verbose:
             print(f"[build] linked {out.relative_to(REPO)}", flush=True)
+    return out
+
+
+MIXER_FLAGS = NO_PK_F32
+
+
+def build_mixers(force: bool = False, jobs: int = 8, verbose: bool = True) -> Path:
+    """``_C_mixers.so``: csrc/mixers/*.hip + csrc/mixers/bindings.cpp."""
+    src = CSRC / "mixers"
+    headers = sorted((CSRC / "include").glob("*.h")) + sorted(src.glob("*.h"))
+    bdir = BUILD / "mixers"
+    kflags = [HIPCC, f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC",
+              f"-I{CSRC / 'include'}", f"-I{src}"] + MIXER_FLAGS
+    tflags, ldflags = _torch_flags()
+    tflags = [f for f in tflags if not f.startswith("-DTORCH_EXTENSION_NAME=")] + \
+        ["-DTORCH_EXTENSION_NAME=_C_mixers"]
+    bflags = [HIPCC, f"--offload-arch={ARCH}"] + tflags + [f"-I{CSRC / 'include'}", f"-I{src}"] \
+        + MIXER_FLAGS
+    jobs_list = [(k, bdir / (k.stem + ".o"), kflags, headers) for k in sorted(src.glob("*.hip"))]
+    jobs_list.append((src / "bindings.cpp", bdir / "bindings.o", bflags + ["-x", "hip"], headers))
+    changed = False
+    with cf.ThreadPoolExecutor(max_workers=max(1, jobs)) as ex:
+        futs = {ex.submit(_compile, s, o, c, d, force): s for s, o, c, d in jobs_list}
+        for f in cf.as_completed(futs):
+            if f.result():
+                changed = True
+                if verbose:
+                    print(f"[build] compiled mixers/{futs[f].name}", flush=True, file=sys.stderr)
+    out = PKG_DIR / ("_C_mixers" + _ext_suffix())
+    if changed or force or not out.exists():
+        _run([HIPCC, f"--offload-arch={ARCH}", "-shared", "-fPIC",
+              *[str(o) for _, o, _, _ in jobs_list], "-o", str(out), *ldflags])
+        if verbose:
+            print(f"[build] linked {out.relative_to(REPO)}", flush=True, file=sys.stderr)
     return out
 
 
@@ -169,6 +212,7 @@ def build_runtime(force: bool = False, jobs: int = 8, verbose: bool = True) -> P
 def build_all(force: bool = False, jobs: int = 8, verbose: bool = True, checked: bool = True):
     """Runtime, release kernels and (``checked``) the bounds-checked kernel build."""
     rt = build_runtime(force=force, jobs=jobs, verbose=verbose)
+    build_mixers(force=force, jobs=jobs, verbose=verbose)
     k = build_kernels(force=force, jobs=jobs, verbose=verbose)
     if checked:
         build_kernels(force=force, jobs=jobs, verbose=verbose, checked=True)
@@ -179,7 +223,7 @@ def main(argv=None):
     ap = argparse.ArgumentParser(description=__doc__)
     ap.add_argument("--force", action="store_true")
     ap.add_argument("-j", "--jobs", type=int, default=min(8, os.cpu_count() or 4))
-    ap.add_argument("--only", choices=["kernels", "checked", "runtime"], default=None)
+    ap.add_argument("--only", choices=["kernels", "checked", "runtime", "mixers"], default=None)
     a = ap.parse_args(argv)
     if a.only == "kernels":
         build_kernels(a.force, a.jobs)
@@ -187,6 +231,8 @@ def main(argv=None):
         build_kernels(a.force, a.jobs, checked=True)
     elif a.only == "runtime":
         build_runtime(a.force, a.jobs)
+    elif a.only == "mixers":
+        build_mixers(a.force, a.jobs)
     else:
         build_all(a.force, a.jobs)
     return 0

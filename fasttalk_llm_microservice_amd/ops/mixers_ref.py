@@ -1,0 +1,207 @@
+"""PyTorch implementations of the sequence-mixer / MoE ops (the CPU backend of
+:mod:`.mixers`, and the semantics the HIP kernels in ``csrc/mixers`` must match).
+
+Everything that the kernels keep in fp32 is fp32 here as well: the residual stream,
+norm statistics, rotary angles, attention scores and weights, the recurrent state and
+all gates and decays that enter the recurrence.  Outputs that feed a matrix product
+are rounded once to the requested storage dtype.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+import torch.nn.functional as F
+
+
+def embed_rows(ids, table):
+    return table.index_select(0, ids.long()).float()
+
+
+def _rms(x, eps):
+    return x * torch.rsqrt((x * x).mean(-1, keepdim=True) + eps)
+
+
+def rms_norm_rows(x, w, eps, out_dtype, add_vec=None):
+    if add_vec is not None:
+        x.add_(add_vec.float())
+    return (_rms(x, eps) * w.float()).to(out_dtype)
+
+
+def add_rms_norm_rows(residual, y, wb, eps, add_vec, next_w, out_dtype, want_cast):
+    residual.add_(_rms(y.float(), eps) * wb.float())
+    if add_vec is not None:
+        residual.add_(add_vec.float())
+    out = (_rms(residual, eps) * next_w.float()).to(out_dtype) if next_w is not None else None
+    cast = residual.to(out_dtype) if want_cast else None
+    return out, cast
+
+
+def rope_table(max_pos: int, dims: int, base: float, device=None):
+    """fp32 [max_pos, dims] = [cos | sin]; frequencies, angles and their cos / sin are
+    all evaluated in fp32 (angle = float(p) * f_i, f_i = base^(-2i/dims))."""
+    i = torch.arange(dims // 2, dtype=torch.float32)
+    f = torch.tensor(float(base), dtype=torch.float32) ** (-2.0 * i / dims)
+    a = torch.arange(max_pos, dtype=torch.float32)[:, None] * f[None]
+    return torch.cat([a.cos(), a.sin()], -1).to(device)
+
+
+def _rope(x, cs, dims):
+    """x [..., T, n] fp32 with cs [T, dims]; rotates the first ``dims`` of n."""
+    half = dims // 2
+    cos, sin = cs[:, :half], cs[:, half:]
+    u, v = x[..., :half], x[..., half:dims]
+    return torch.cat([u * cos - v * sin, v * cos + u * sin, x[..., dims:]], -1)
+
+
+def short_conv_silu(x, conv_w, conv_state, seg):
+    t, c = x.shape
+    taps = conv_w.shape[1]
+    out = torch.empty_like(x)
+    w = conv_w.float()
+    start = seg.start.tolist()
+    for s in range(seg.num):
+        a, b = start[s], start[s + 1]
+        slot = int(seg.slot[s])
+        if slot < 0 or b == a:
+            out[a:b] = 0
+            continue
+        hist = conv_state[slot] if int(seg.pos0[s]) > 0 else torch.zeros_like(conv_state[slot])
+        xp = torch.cat([hist, x[a:b].float()], 0)            # [taps-1 + n, C]
+        n = b - a
+        y = sum(xp[j:j + n] * w[:, j][None] for j in range(taps))
+        out[a:b] = (y * torch.sigmoid(y)).to(x.dtype)
+        if taps > 1:
+            conv_state[slot] = xp[n:]
+    return out
+
+
+def gated_delta_rule(qkv, a, b, a_log, dt_bias, state, seg, heads, kv_heads, dk, dv):
+    t = qkv.shape[0]
+    rep = heads // kv_heads
+    nq = kv_heads * dk
+    q = qkv[:, :nq].float().view(t, kv_heads, dk)
+    k = qkv[:, nq:2 * nq].float().view(t, kv_heads, dk)
+    v = qkv[:, 2 * nq:].float().view(t, heads, dv)
+    q = q * torch.rsqrt((q * q).sum(-1, keepdim=True) + 1e-6) * dk ** -0.5
+    k = k * torch.rsqrt((k * k).sum(-1, keepdim=True) + 1e-6)
+    beta = torch.sigmoid(b.float())
+    g = torch.exp(-torch.exp(a_log.float())[None, :, None]
+                  * F.softplus(a.float().view(t, heads, dk) + dt_bias.float().view(heads, dk)))
+    o = torch.zeros(t, heads, dv, dtype=torch.float32, device=qkv.device)
+    start = seg.start.tolist()
+    for s in range(seg.num):
+        slot = int(seg.slot[s])
+        if slot < 0:
+            continue
+        S = state[slot] if int(seg.pos0[s]) > 0 else torch.zeros_like(state[slot])
+        for r in range(start[s], start[s + 1]):
+            qt = q[r].repeat_interleave(rep, 0)
+            kt = k[r].repeat_interleave(rep, 0)
+            S = g[r][:, :, None] * S
+            u = beta[r][:, None] * (v[r] - torch.einsum("hkv,hk->hv", S, kt))
+            S = S + kt[:, :, None] * u[:, None, :]
+            o[r] = torch.einsum("hkv,hk->hv", S, qt)
+        state[slot] = S
+    return o.view(t, heads * dv)
+
+
+def head_rms_gate(o, w, gate_pre, eps, heads, dv, out_dtype):
+    t = o.shape[0]
+    x = o.view(t, heads, dv)
+    y = _rms(x, eps) * w.float() * torch.sigmoid(gate_pre.float().view(t, heads, dv))
+    return y.view(t, heads * dv).to(out_dtype)
+
+
+def latent_kv_write(dkv, norm_w, eps, table, rot_dims, positions, slot_mapping, cache, rank):
+    t = dkv.shape[0]
+    if t == 0:
+        return
+    x = dkv.float()
+    c = _rms(x[:, :rank], eps) * norm_w.float()
+    kr = _rope(x[:, rank:], table[positions.long()], rot_dims)
+    row = torch.cat([c, kr], -1).to(cache.dtype)
+    slots = slot_mapping[:t].long()
+    keep = slots >= 0
+    if keep.any():
+        cache.view(-1, cache.shape[-1])[slots[keep]] = row[keep]
+
+
+def latent_q_rope(q, table, rot_dims, positions, heads, dn, dr):
+    """q [T, heads*(dn+dr)] -> (q_unrotated fp32 [T, heads, dn], q_rotated fp32 [T, heads, dr])."""
+    t = q.shape[0]
+    x = q.float().view(t, heads, dn + dr)
+    cs = table[positions.long()]
+    return x[..., :dn].contiguous(), _rope(x[..., dn:].transpose(0, 1), cs, rot_dims).transpose(0, 1).contiguous()
+
+
+def latent_attention(qa, qr, cache, seg, scale, rank):
+    """qa fp32 [heads, T, rank] (queries in latent space) and qr fp32 [T, heads, dr]
+    (rotated part) against cache rows [c (rank) | rotated key (dr)]; returns the
+    softmax-weighted sums of the c rows, fp32 [heads, T, rank]."""
+    heads, t, _ = qa.shape
+    out = torch.zeros(heads, t, rank, dtype=torch.float32, device=qa.device)
+    bs = cache.shape[1]
+    start = seg.start.tolist()
+    for s in range(seg.num):
+        a, b = start[s], start[s + 1]
+        n = int(seg.kv_len[s])
+        if b == a or n == 0:
+            continue
+        nblk = (n + bs - 1) // bs
+        kv = cache[seg.block_tables[s, :nblk].long()].reshape(nblk * bs, -1)[:n].float()
+        sc = (torch.einsum("htd,jd->htj", qa[:, a:b], kv[:, :rank])
+              + torch.einsum("thd,jd->htj", qr[a:b], kv[:, rank:])) * scale
+        qpos = int(seg.pos0[s]) + torch.arange(b - a, device=qa.device)
+        mask = torch.arange(n, device=qa.device)[None, :] <= qpos[:, None]
+        sc = sc.masked_fill(~mask[None], float("-inf"))
+        p = torch.softmax(sc, -1)
+        out[:, a:b] = torch.einsum("htj,jr->htr", p, kv[:, :rank])
+    return out
+
+
+def moe_topk(z, correction, top, groups, keep):
+    s = torch.softmax(z.float(), -1)
+    ch = s + correction.float()
+    e = z.shape[1]
+    if groups > 1 and keep < groups:
+        gs = ch.view(-1, groups, e // groups).max(-1).values
+        kg = gs.topk(keep, -1).indices
+        gm = torch.zeros_like(gs, dtype=torch.bool).scatter_(1, kg, True)
+        ch = ch.masked_fill(~gm.repeat_interleave(e // groups, 1), float("-inf"))
+    idx = ch.topk(top, -1).indices
+    return idx.int(), s.gather(1, idx)
+
+
+def clamp_swiglu(gu, limit, rows_scale=None):
+    """gu [n, 2*ff (+1)] = [gate | up (| per-row gate logit)] -> y [n, ff]:
+    g = min(gate, limit), u = clamp(up, +-limit), y = g * sigmoid(1.702 g) * (u + 1)."""
+    ff = gu.shape[1] // 2
+    g = gu[:, :ff].float().clamp(max=limit)
+    u = gu[:, ff:2 * ff].float().clamp(-limit, limit)
+    return (g * torch.sigmoid(1.702 * g) * (u + 1)).to(gu.dtype)
+
+
+def relu_sq(x):
+    r = torch.relu(x.float())
+    return (r * r).to(x.dtype)
+
+
+def gelu_tanh(z):
+    return 0.5 * z * (1 + torch.tanh(math.sqrt(2 / math.pi) * (z + 0.044715 * z * z * z)))
+
+
+def side_gate(gpre, table, ids, col0, sd):
+    e = table.index_select(0, ids.long())[:, col0:col0 + sd].float()
+    return (gelu_tanh(gpre.float()) * e).to(gpre.dtype)
+
+
+def scale_add_rows(out, y, rows, weights, sigmoid: bool):
+    w = weights.float()
+    if sigmoid:
+        w = torch.sigmoid(w)
+    upd = y.float() * w[:, None]
+    if rows is None:
+        out.add_(upd)
+    else:
+        out.index_add_(0, rows.long(), upd)
