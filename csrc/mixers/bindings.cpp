@@ -1,0 +1,313 @@
+// PyTorch bindings of the sequence-mixer / MoE kernels (extension `_C_mixers`).
+//
+// As in csrc/bindings.cpp every op validates dtype / device / shape on the host (a
+// mis-shaped launch of a hand-written kernel can fault the GPU) and launches on the
+// caller's current stream without allocating or synchronising.
+#include <torch/extension.h>
+#include <c10/hip/HIPStream.h>
+#include <hip/hip_runtime.h>
+
+extern "C" {
+int mx_embed_rows(float* out, const int* ids, const void* table, int bf16, int rows, int width, int vocab,
+                  hipStream_t s);
+int mx_add_rms_norm(float* x, const void* y, int y_bf16, long y_stride, const float* wb, const float* add_vec,
+                    const float* next_w, void* out, void* cast, int out_bf16, int rows, int width, float eps,
+                    hipStream_t s);
+int mx_head_rms_gate(void* out, int out_bf16, const float* o, const float* w, const void* gate, int gate_bf16,
+                     long gate_stride, long rows, int heads, int dv, float eps, hipStream_t s);
+int mx_relu_sq(void* x, int bf16, long n, hipStream_t s);
+int mx_clamp_swiglu(void* out, const void* gu, int bf16, long gu_stride, long rows, int ff, float limit,
+                    hipStream_t s);
+int mx_side_gate(void* out, const void* gpre, const void* table, int bf16, long table_stride, const int* ids,
+                 int col0, long rows, int sd, int vocab, hipStream_t s);
+int mx_scale_add_rows(float* out, const void* y, int y_bf16, const int* rows, const void* weights, int w_bf16,
+                      int sigmoid, long n, int width, int out_rows, hipStream_t s);
+int mx_short_conv_silu(void* out, const void* x, int bf16, const float* w, float* hist, const int* start,
+                       const int* pos0, const int* slot, int num_segs, int max_rows, int channels, int taps,
+                       int num_slots, hipStream_t s);
+int mx_delta_prep(float* qn, float* kn, float* g, float* beta, const void* qkv, int bf16, long qkv_stride,
+                  const void* a, long a_stride, const void* b, long b_stride, const float* a_log,
+                  const float* dt_bias, long rows, int heads, int kv_heads, int dk, hipStream_t s);
+int mx_delta_max_dk();
+int mx_delta_rule(float* o, const float* qn, const float* kn, const float* g, const float* beta,
+                  const void* qkv, int bf16, long qkv_stride, float* state, const int* start, const int* pos0,
+                  const int* slot, int num_segs, int heads, int kv_heads, int dk, int dv, int num_slots,
+                  hipStream_t s);
+int mx_latent_kv_write(const void* dkv, int bf16, long stride, const float* w, float eps, const float* table,
+                       int table_rows, int dims, const int* positions, const int* slots, void* cache,
+                       int cache_bf16, long num_slots, long rows, int rank, int dr, hipStream_t s);
+int mx_latent_q_rope(float* qn, float* qr, const void* q, int bf16, long stride, const float* table,
+                     int table_rows, int dims, const int* positions, long rows, int heads, int dn, int dr,
+                     hipStream_t s);
+int mx_latent_max_rank();
+int mx_latent_attention(float* out, const float* qa, const float* qr, const void* cache, int cache_bf16,
+                        const int* start, const int* pos0, const int* kv_len, const int* bt, int bt_stride,
+                        int num_segs, int max_rows, int heads, long total_rows, int rank, int dr,
+                        int block_size, int num_blocks, float scale, hipStream_t s);
+int mx_moe_topk(int* idx, float* wts, const float* z, const float* corr, long rows, int experts, int top,
+                int groups, int keep, hipStream_t s);
+}
+
+namespace {
+
+using at::Tensor;
+using OptT = c10::optional<Tensor>;
+
+hipStream_t stream() { return c10::hip::getCurrentHIPStream().stream(); }
+
+bool is_act(const Tensor& t) { return t.scalar_type() == at::kFloat || t.scalar_type() == at::kBFloat16; }
+int bf(const Tensor& t) { return t.scalar_type() == at::kBFloat16 ? 1 : 0; }
+
+void chk(int rc, const char* what) { TORCH_CHECK(rc == 0, what, " failed (", rc, ")"); }
+
+void check_f32(const Tensor& t, const char* n) {
+  TORCH_CHECK(t.is_cuda() && t.scalar_type() == at::kFloat && t.is_contiguous(), n, ": fp32 contiguous GPU tensor");
+}
+void check_i32(const Tensor& t, const char* n) {
+  TORCH_CHECK(t.is_cuda() && t.scalar_type() == at::kInt && t.is_contiguous(), n, ": int32 contiguous GPU tensor");
+}
+// 2-D rows with unit inner stride (views of a wider product are fine)
+void check_rows(const Tensor& t, const char* n) {
+  TORCH_CHECK(t.is_cuda() && is_act(t) && t.dim() == 2 && (t.size(1) == 1 || t.stride(1) == 1), n,
+              ": 2-D fp32/bf16 GPU rows with unit inner stride");
+}
+
+// segment arrays: start [S+1], pos0 / slot / kv_len [>= S]
+void check_segs(const Tensor& start, const Tensor& a, const Tensor& b, int64_t num) {
+  check_i32(start, "seg.start");
+  check_i32(a, "seg array");
+  check_i32(b, "seg array");
+  TORCH_CHECK(num >= 0 && start.numel() >= num + 1 && a.numel() >= num && b.numel() >= num, "segment arrays too short");
+}
+
+void embed_rows(Tensor out, Tensor ids, Tensor table) {
+  check_f32(out, "out");
+  check_i32(ids, "ids");
+  TORCH_CHECK(table.is_cuda() && is_act(table) && table.is_contiguous() && table.dim() == 2, "table");
+  TORCH_CHECK(out.dim() == 2 && out.size(0) == ids.numel() && out.size(1) == table.size(1), "out shape");
+  chk(mx_embed_rows(out.data_ptr<float>(), ids.data_ptr<int>(), table.data_ptr(), bf(table), (int)ids.numel(),
+                    (int)table.size(1), (int)table.size(0), stream()), "embed_rows");
+}
+
+void add_rms_norm(Tensor x, OptT y, OptT wb, OptT add_vec, OptT next_w, OptT out, OptT cast, double eps) {
+  check_f32(x, "residual");
+  TORCH_CHECK(x.dim() == 2, "residual 2-D");
+  const int64_t rows = x.size(0), width = x.size(1);
+  const void* yp = nullptr;
+  int ybf = 0;
+  long ys = 0;
+  if (y) {
+    check_rows(*y, "y");
+    TORCH_CHECK(y->size(0) == rows && y->size(1) == width && wb, "y shape / wb");
+    check_f32(*wb, "wb");
+    TORCH_CHECK(wb->numel() == width, "wb size");
+    yp = y->data_ptr();
+    ybf = bf(*y);
+    ys = y->stride(0);
+  }
+  if (add_vec) { check_f32(*add_vec, "add_vec"); TORCH_CHECK(add_vec->numel() == width, "add_vec size"); }
+  TORCH_CHECK((bool)next_w == (bool)out, "next_w and out go together");
+  int obf = 0;
+  if (out) {
+    check_f32(*next_w, "next_w");
+    TORCH_CHECK(next_w->numel() == width && out->is_cuda() && is_act(*out) && out->is_contiguous() &&
+                out->numel() == rows * width, "out");
+    obf = bf(*out);
+  }
+  if (cast) {
+    TORCH_CHECK(cast->is_cuda() && is_act(*cast) && cast->is_contiguous() && cast->numel() == rows * width, "cast");
+    TORCH_CHECK(!out || bf(*cast) == obf, "out and cast share a dtype");
+    obf = bf(*cast);
+  }
+  chk(mx_add_rms_norm(x.data_ptr<float>(), yp, ybf, ys, wb ? wb->data_ptr<float>() : nullptr,
+                      add_vec ? add_vec->data_ptr<float>() : nullptr, next_w ? next_w->data_ptr<float>() : nullptr,
+                      out ? out->data_ptr() : nullptr, cast ? cast->data_ptr() : nullptr, obf, (int)rows,
+                      (int)width, (float)eps, stream()), "add_rms_norm");
+}
+
+void head_rms_gate(Tensor out, Tensor o, Tensor w, Tensor gate, double eps, int64_t heads, int64_t dv) {
+  check_f32(o, "o");
+  check_f32(w, "w");
+  check_rows(gate, "gate");
+  TORCH_CHECK(o.dim() == 2 && o.size(1) == heads * dv && w.numel() == dv && gate.size(0) == o.size(0) &&
+              gate.size(1) == heads * dv, "head_rms_gate shapes");
+  TORCH_CHECK(out.is_cuda() && is_act(out) && out.is_contiguous() && out.sizes() == o.sizes() &&
+              bf(out) == bf(gate), "out");
+  chk(mx_head_rms_gate(out.data_ptr(), bf(out), o.data_ptr<float>(), w.data_ptr<float>(), gate.data_ptr(),
+                       bf(gate), gate.stride(0), o.size(0), (int)heads, (int)dv, (float)eps, stream()),
+      "head_rms_gate");
+}
+
+void relu_sq(Tensor x) {
+  TORCH_CHECK(x.is_cuda() && is_act(x) && x.is_contiguous(), "x");
+  chk(mx_relu_sq(x.data_ptr(), bf(x), x.numel(), stream()), "relu_sq");
+}
+
+void clamp_swiglu(Tensor out, Tensor gu, double limit) {
+  check_rows(gu, "gu");
+  const int64_t ff = gu.size(1) / 2;
+  TORCH_CHECK(out.is_cuda() && out.is_contiguous() && out.scalar_type() == gu.scalar_type() && out.dim() == 2 &&
+              out.size(0) == gu.size(0) && out.size(1) == ff && ff >= 1, "out");
+  chk(mx_clamp_swiglu(out.data_ptr(), gu.data_ptr(), bf(gu), gu.stride(0), gu.size(0), (int)ff, (float)limit,
+                      stream()), "clamp_swiglu");
+}
+
+void side_gate(Tensor out, Tensor gpre, Tensor table, Tensor ids, int64_t col0) {
+  check_i32(ids, "ids");
+  TORCH_CHECK(gpre.is_cuda() && is_act(gpre) && gpre.is_contiguous() && gpre.dim() == 2, "gpre");
+  TORCH_CHECK(out.is_cuda() && out.is_contiguous() && out.scalar_type() == gpre.scalar_type() &&
+              out.sizes() == gpre.sizes(), "out");
+  TORCH_CHECK(table.is_cuda() && table.is_contiguous() && table.dim() == 2 &&
+              table.scalar_type() == gpre.scalar_type() && col0 >= 0 && col0 + gpre.size(1) <= table.size(1) &&
+              ids.numel() == gpre.size(0), "table / ids");
+  chk(mx_side_gate(out.data_ptr(), gpre.data_ptr(), table.data_ptr(), bf(gpre), table.size(1),
+                   ids.data_ptr<int>(), (int)col0, gpre.size(0), (int)gpre.size(1), (int)table.size(0), stream()),
+      "side_gate");
+}
+
+void scale_add_rows(Tensor out, Tensor y, OptT rows, Tensor weights, bool sigmoid) {
+  check_f32(out, "out");
+  TORCH_CHECK(y.is_cuda() && is_act(y) && y.is_contiguous() && y.dim() == 2 && out.dim() == 2 &&
+              y.size(1) == out.size(1), "y");
+  TORCH_CHECK(weights.is_cuda() && is_act(weights) && weights.is_contiguous() && weights.numel() == y.size(0),
+              "weights");
+  if (rows) { check_i32(*rows, "rows"); TORCH_CHECK(rows->numel() == y.size(0), "rows size"); }
+  else TORCH_CHECK(y.size(0) == out.size(0), "identity rows need equal row counts");
+  chk(mx_scale_add_rows(out.data_ptr<float>(), y.data_ptr(), bf(y), rows ? rows->data_ptr<int>() : nullptr,
+                        weights.data_ptr(), bf(weights), sigmoid ? 1 : 0, y.size(0), (int)y.size(1),
+                        (int)out.size(0), stream()), "scale_add_rows");
+}
+
+void short_conv_silu(Tensor out, Tensor x, Tensor w, Tensor hist, Tensor start, Tensor pos0, Tensor slot,
+                     int64_t num_segs, int64_t max_rows) {
+  TORCH_CHECK(x.is_cuda() && is_act(x) && x.is_contiguous() && x.dim() == 2, "x");
+  TORCH_CHECK(out.is_cuda() && out.is_contiguous() && out.scalar_type() == x.scalar_type() &&
+              out.sizes() == x.sizes(), "out");
+  check_f32(w, "conv_w");
+  check_f32(hist, "conv_state");
+  const int64_t c = x.size(1), taps = w.size(1);
+  TORCH_CHECK(w.dim() == 2 && w.size(0) == c && hist.dim() == 3 && hist.size(1) == taps - 1 && hist.size(2) == c,
+              "conv shapes");
+  check_segs(start, pos0, slot, num_segs);
+  TORCH_CHECK(max_rows <= x.size(0), "max_rows");
+  chk(mx_short_conv_silu(out.data_ptr(), x.data_ptr(), bf(x), w.data_ptr<float>(), hist.data_ptr<float>(),
+                         start.data_ptr<int>(), pos0.data_ptr<int>(), slot.data_ptr<int>(), (int)num_segs,
+                         (int)max_rows, (int)c, (int)taps, (int)hist.size(0), stream()), "short_conv_silu");
+}
+
+void gated_delta_rule(Tensor o, Tensor qkv, Tensor a, Tensor b, Tensor a_log, Tensor dt_bias, Tensor state,
+                      Tensor start, Tensor pos0, Tensor slot, int64_t num_segs, int64_t heads, int64_t kv_heads,
+                      int64_t dk, int64_t dv) {
+  check_f32(o, "o");
+  check_rows(qkv, "qkv");
+  check_rows(a, "a");
+  check_rows(b, "b");
+  check_f32(a_log, "a_log");
+  check_f32(dt_bias, "dt_bias");
+  check_f32(state, "state");
+  const int64_t t = qkv.size(0);
+  TORCH_CHECK(heads >= 1 && kv_heads >= 1 && heads % kv_heads == 0 && dk >= 1 && dk <= mx_delta_max_dk() && dv >= 1,
+              "delta rule sizes");
+  TORCH_CHECK(qkv.size(1) == 2 * kv_heads * dk + heads * dv && a.size(0) == t && a.size(1) == heads * dk &&
+              b.size(0) == t && b.size(1) == heads && a_log.numel() == heads && dt_bias.numel() == heads * dk &&
+              o.numel() == t * heads * dv && a.scalar_type() == qkv.scalar_type() &&
+              b.scalar_type() == qkv.scalar_type(), "delta rule shapes");
+  TORCH_CHECK(state.dim() == 4 && state.size(1) == heads && state.size(2) == dk && state.size(3) == dv, "state");
+  check_segs(start, pos0, slot, num_segs);
+  auto f32 = qkv.options().dtype(at::kFloat);
+  Tensor qn = at::empty({t, kv_heads, dk}, f32), kn = at::empty({t, kv_heads, dk}, f32);
+  Tensor g = at::empty({t, heads, dk}, f32), beta = at::empty({t, heads}, f32);
+  chk(mx_delta_prep(qn.data_ptr<float>(), kn.data_ptr<float>(), g.data_ptr<float>(), beta.data_ptr<float>(),
+                    qkv.data_ptr(), bf(qkv), qkv.stride(0), a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0),
+                    a_log.data_ptr<float>(), dt_bias.data_ptr<float>(), t, (int)heads, (int)kv_heads, (int)dk,
+                    stream()), "delta_prep");
+  chk(mx_delta_rule(o.data_ptr<float>(), qn.data_ptr<float>(), kn.data_ptr<float>(), g.data_ptr<float>(),
+                    beta.data_ptr<float>(), qkv.data_ptr(), bf(qkv), qkv.stride(0), state.data_ptr<float>(),
+                    start.data_ptr<int>(), pos0.data_ptr<int>(), slot.data_ptr<int>(), (int)num_segs, (int)heads,
+                    (int)kv_heads, (int)dk, (int)dv, (int)state.size(0), stream()), "delta_rule");
+}
+
+void latent_kv_write(Tensor dkv, Tensor w, double eps, Tensor table, int64_t dims, Tensor positions,
+                     Tensor slots, Tensor cache, int64_t rank) {
+  check_rows(dkv, "dkv");
+  check_f32(w, "norm_w");
+  check_f32(table, "rope table");
+  check_i32(positions, "positions");
+  check_i32(slots, "slot_mapping");
+  const int64_t t = dkv.size(0), dr = dkv.size(1) - rank;
+  TORCH_CHECK(rank >= 1 && dr >= 0 && dims % 2 == 0 && dims <= dr && w.numel() == rank && table.dim() == 2 &&
+              table.size(1) == dims && positions.numel() >= t && slots.numel() >= t, "latent_kv_write shapes");
+  TORCH_CHECK(cache.is_cuda() && cache.is_contiguous() && cache.dim() == 3 && cache.size(2) == rank + dr &&
+              cache.scalar_type() == dkv.scalar_type(), "cache");
+  chk(mx_latent_kv_write(dkv.data_ptr(), bf(dkv), dkv.stride(0), w.data_ptr<float>(), (float)eps,
+                         table.data_ptr<float>(), (int)table.size(0), (int)dims, positions.data_ptr<int>(),
+                         slots.data_ptr<int>(), cache.data_ptr(), bf(cache), cache.size(0) * cache.size(1), t,
+                         (int)rank, (int)dr, stream()), "latent_kv_write");
+}
+
+void latent_q_rope(Tensor qn, Tensor qr, Tensor q, Tensor table, int64_t dims, Tensor positions, int64_t heads,
+                   int64_t dn, int64_t dr) {
+  check_f32(qn, "qn");
+  check_f32(qr, "qr");
+  check_rows(q, "q");
+  check_f32(table, "rope table");
+  check_i32(positions, "positions");
+  const int64_t t = q.size(0);
+  TORCH_CHECK(q.size(1) == heads * (dn + dr) && qn.numel() == t * heads * dn && qr.numel() == t * heads * dr &&
+              dims % 2 == 0 && dims <= dr && table.dim() == 2 && table.size(1) == dims && positions.numel() >= t,
+              "latent_q_rope shapes");
+  chk(mx_latent_q_rope(qn.data_ptr<float>(), qr.data_ptr<float>(), q.data_ptr(), bf(q), q.stride(0),
+                       table.data_ptr<float>(), (int)table.size(0), (int)dims, positions.data_ptr<int>(), t,
+                       (int)heads, (int)dn, (int)dr, stream()), "latent_q_rope");
+}
+
+void latent_attention(Tensor out, Tensor qa, Tensor qr, Tensor cache, Tensor start, Tensor pos0, Tensor kv_len,
+                      Tensor bt, int64_t num_segs, int64_t max_rows, double scale, int64_t rank) {
+  check_f32(out, "out");
+  check_f32(qa, "qa");
+  check_f32(qr, "qr");
+  TORCH_CHECK(qa.dim() == 3 && qr.dim() == 3 && qa.size(2) == rank && out.sizes() == qa.sizes(), "qa / out");
+  const int64_t heads = qa.size(0), t = qa.size(1), dr = qr.size(2);
+  TORCH_CHECK(qr.size(0) == t && qr.size(1) == heads && rank <= mx_latent_max_rank(), "qr");
+  TORCH_CHECK(cache.is_cuda() && cache.is_contiguous() && cache.dim() == 3 && cache.size(2) == rank + dr &&
+              is_act(cache), "cache");
+  check_segs(start, pos0, kv_len, num_segs);
+  check_i32(bt, "block tables");
+  TORCH_CHECK(bt.dim() == 2 && bt.size(0) >= num_segs && max_rows <= t, "block tables / max_rows");
+  chk(mx_latent_attention(out.data_ptr<float>(), qa.data_ptr<float>(), qr.data_ptr<float>(), cache.data_ptr(),
+                          bf(cache), start.data_ptr<int>(), pos0.data_ptr<int>(), kv_len.data_ptr<int>(),
+                          bt.data_ptr<int>(), (int)bt.size(1), (int)num_segs, (int)max_rows, (int)heads, t,
+                          (int)rank, (int)dr, (int)cache.size(1), (int)cache.size(0), (float)scale, stream()),
+      "latent_attention");
+}
+
+void moe_topk(Tensor idx, Tensor wts, Tensor z, Tensor corr, int64_t top, int64_t groups, int64_t keep) {
+  check_i32(idx, "idx");
+  check_f32(wts, "wts");
+  check_f32(z, "z");
+  check_f32(corr, "correction");
+  TORCH_CHECK(z.dim() == 2 && corr.numel() == z.size(1) && idx.numel() == z.size(0) * top &&
+              wts.numel() == z.size(0) * top, "moe_topk shapes");
+  chk(mx_moe_topk(idx.data_ptr<int>(), wts.data_ptr<float>(), z.data_ptr<float>(), corr.data_ptr<float>(),
+                  z.size(0), (int)z.size(1), (int)top, (int)groups, (int)keep, stream()), "moe_topk");
+}
+
+}  // namespace
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+  m.def("embed_rows", &embed_rows);
+  m.def("add_rms_norm", &add_rms_norm);
+  m.def("head_rms_gate", &head_rms_gate);
+  m.def("relu_sq", &relu_sq);
+  m.def("clamp_swiglu", &clamp_swiglu);
+  m.def("side_gate", &side_gate);
+  m.def("scale_add_rows", &scale_add_rows);
+  m.def("short_conv_silu", &short_conv_silu);
+  m.def("gated_delta_rule", &gated_delta_rule);
+  m.def("latent_kv_write", &latent_kv_write);
+  m.def("latent_q_rope", &latent_q_rope);
+  m.def("latent_attention", &latent_attention);
+  m.def("moe_topk", &moe_topk);
+  m.def("delta_max_dk", []() { return (int64_t)mx_delta_max_dk(); });
+  m.def("latent_max_rank", []() { return (int64_t)mx_latent_max_rank(); });
+}

@@ -1,0 +1,233 @@
+// Row-wise kernels around an fp32 residual stream: embedding rows, the fused
+// "post-norm add + next pre-norm" step, per-head gated output norm, activations
+// (relu^2, clamped GLU, gelu * token-side embedding) and the weighted row scatter-add
+// that combines expert outputs.
+#include "mx_common.h"
+
+namespace mx {
+
+template <typename T>
+__global__ void embed_rows_kernel(float* __restrict__ out, const int* __restrict__ ids,
+                                  const T* __restrict__ table, int width, int vocab) {
+  const int row = blockIdx.x;
+  int id = ids[row];
+  if (id < 0 || id >= vocab) id = 0;
+  for (int i = threadIdx.x; i < width; i += blockDim.x)
+    out[(long)row * width + i] = ld(table, (long)id * width + i);
+}
+
+// residual (fp32, in place): x += rms_norm(y) * wb (+ add_vec);
+// out = rms_norm(x) * next_w (TO);  cast = x (TO).  Every part is optional.
+template <typename TY, typename TO, int NT>
+__global__ void add_rms_norm_kernel(float* __restrict__ x, const TY* __restrict__ y, long y_stride,
+                                    const float* __restrict__ wb, const float* __restrict__ add_vec,
+                                    const float* __restrict__ next_w, TO* __restrict__ out,
+                                    TO* __restrict__ cast, int width, float eps) {
+  __shared__ float red[NT / 64];
+  const long row = blockIdx.x;
+  float* xr = x + row * width;
+  if (y != nullptr) {
+    const TY* yr = y + row * y_stride;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < width; i += NT) {
+      const float v = ld(yr, i);
+      ss += v * v;
+    }
+    ss = block_sum<NT>(ss, red);
+    const float r = 1.0f / sqrtf(ss / (float)width + eps);
+    for (int i = threadIdx.x; i < width; i += NT) {
+      float v = xr[i] + ld(yr, i) * r * wb[i];
+      if (add_vec != nullptr) v += add_vec[i];
+      xr[i] = v;
+    }
+  } else if (add_vec != nullptr) {
+    for (int i = threadIdx.x; i < width; i += NT) xr[i] += add_vec[i];
+  }
+  // each thread re-reads only what it wrote itself: no barrier needed
+  if (out != nullptr) {
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < width; i += NT) {
+      const float v = xr[i];
+      ss += v * v;
+    }
+    ss = block_sum<NT>(ss, red);
+    const float r = 1.0f / sqrtf(ss / (float)width + eps);
+    for (int i = threadIdx.x; i < width; i += NT) st(out, row * width + i, xr[i] * r * next_w[i]);
+  }
+  if (cast != nullptr)
+    for (int i = threadIdx.x; i < width; i += NT) st(cast, row * width + i, xr[i]);
+}
+
+// one wave per (row, head): out = o / rms(o) * w * sigmoid(gate)
+template <typename TG, typename TO>
+__global__ void head_rms_gate_kernel(TO* __restrict__ out, const float* __restrict__ o,
+                                     const float* __restrict__ w, const TG* __restrict__ gate,
+                                     long gate_stride, long pairs, int heads, int dv, float eps) {
+  const long pair = (long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (pair >= pairs) return;
+  const int lane = threadIdx.x & 63;
+  const long row = pair / heads;
+  const int h = (int)(pair % heads);
+  const float* op = o + (row * heads + h) * dv;
+  float ss = 0.f;
+  for (int i = lane; i < dv; i += 64) ss += op[i] * op[i];
+  ss = ft::wave_sum(ss);
+  const float r = 1.0f / sqrtf(ss / (float)dv + eps);
+  for (int i = lane; i < dv; i += 64) {
+    const float g = sigmoidf_(ld(gate, row * gate_stride + (long)h * dv + i));
+    st(out, (row * heads + h) * dv + i, op[i] * r * w[i] * g);
+  }
+}
+
+template <typename T>
+__global__ void relu_sq_kernel(T* __restrict__ x, long n) {
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) {
+    const float v = fmaxf(ld(x, i), 0.f);
+    st(x, i, v * v);
+  }
+}
+
+// rows [gate (ff) | up (ff) | ...]: g = min(gate, limit), u = clamp(up, +-limit),
+// out = g * sigmoid(1.702 g) * (u + 1)
+template <typename T>
+__global__ void clamp_swiglu_kernel(T* __restrict__ out, const T* __restrict__ gu, long gu_stride,
+                                    long rows, int ff, float limit) {
+  const long n = rows * ff;
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) {
+    const long r = i / ff;
+    const int c = (int)(i % ff);
+    const float g = fminf(ld(gu, r * gu_stride + c), limit);
+    const float u = fminf(fmaxf(ld(gu, r * gu_stride + ff + c), -limit), limit);
+    st(out, i, g * sigmoidf_(1.702f * g) * (u + 1.0f));
+  }
+}
+
+__device__ __forceinline__ float gelu_tanh_(float z) {
+  return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+
+template <typename T>
+__global__ void side_gate_kernel(T* __restrict__ out, const T* __restrict__ gpre,
+                                 const T* __restrict__ table, long table_stride,
+                                 const int* __restrict__ ids, int col0, long rows, int sd, int vocab) {
+  const long n = rows * sd;
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) {
+    const long r = i / sd;
+    const int c = (int)(i % sd);
+    int id = ids[r];
+    if (id < 0 || id >= vocab) id = 0;
+    st(out, i, gelu_tanh_(ld(gpre, i)) * ld(table, (long)id * table_stride + col0 + c));
+  }
+}
+
+// out[rows[i]] += w_i * y[i]; rows == nullptr: identity.  No row repeats within a call.
+template <typename TY, typename TW>
+__global__ void scale_add_rows_kernel(float* __restrict__ out, const TY* __restrict__ y,
+                                      const int* __restrict__ rows, const TW* __restrict__ weights,
+                                      int sigmoid, int width, int out_rows) {
+  const long i = blockIdx.x;
+  const long dst = rows != nullptr ? rows[i] : i;
+  if (dst < 0 || dst >= out_rows) return;
+  float w = ld(weights, i);
+  if (sigmoid) w = sigmoidf_(w);
+  for (int c = threadIdx.x; c < width; c += blockDim.x)
+    out[dst * width + c] += w * ld(y, i * width + c);
+}
+
+}  // namespace mx
+
+using namespace mx;
+
+extern "C" int mx_embed_rows(float* out, const int* ids, const void* table, int bf16, int rows,
+                             int width, int vocab, hipStream_t s) {
+  if (rows <= 0) return 0;
+  MX_DISPATCH_T(bf16, hipLaunchKernelGGL((embed_rows_kernel<T>), dim3(rows), dim3(256), 0, s, out, ids,
+                                         (const T*)table, width, vocab));
+  return (int)hipGetLastError();
+}
+
+template <typename TY, typename TO>
+static void launch_add_rms(float* x, const void* y, long ys, const float* wb, const float* av,
+                           const float* nw, void* out, void* cast, int rows, int width, float eps,
+                           hipStream_t s) {
+  hipLaunchKernelGGL((add_rms_norm_kernel<TY, TO, 256>), dim3(rows), dim3(256), 0, s, x, (const TY*)y,
+                     ys, wb, av, nw, (TO*)out, (TO*)cast, width, eps);
+}
+
+extern "C" int mx_add_rms_norm(float* x, const void* y, int y_bf16, long y_stride, const float* wb,
+                               const float* add_vec, const float* next_w, void* out, void* cast,
+                               int out_bf16, int rows, int width, float eps, hipStream_t s) {
+  if (rows <= 0) return 0;
+  if (y_bf16) {
+    if (out_bf16) launch_add_rms<bf16_t, bf16_t>(x, y, y_stride, wb, add_vec, next_w, out, cast, rows, width, eps, s);
+    else launch_add_rms<bf16_t, float>(x, y, y_stride, wb, add_vec, next_w, out, cast, rows, width, eps, s);
+  } else {
+    if (out_bf16) launch_add_rms<float, bf16_t>(x, y, y_stride, wb, add_vec, next_w, out, cast, rows, width, eps, s);
+    else launch_add_rms<float, float>(x, y, y_stride, wb, add_vec, next_w, out, cast, rows, width, eps, s);
+  }
+  return (int)hipGetLastError();
+}
+
+extern "C" int mx_head_rms_gate(void* out, int out_bf16, const float* o, const float* w,
+                                const void* gate, int gate_bf16, long gate_stride, long rows, int heads,
+                                int dv, float eps, hipStream_t s) {
+  const long pairs = rows * heads;
+  if (pairs <= 0) return 0;
+  const dim3 grid((unsigned)((pairs + 3) / 4)), block(256);
+  if (gate_bf16 && out_bf16)
+    hipLaunchKernelGGL((head_rms_gate_kernel<bf16_t, bf16_t>), grid, block, 0, s, (bf16_t*)out, o, w,
+                       (const bf16_t*)gate, gate_stride, pairs, heads, dv, eps);
+  else if (!gate_bf16 && !out_bf16)
+    hipLaunchKernelGGL((head_rms_gate_kernel<float, float>), grid, block, 0, s, (float*)out, o, w,
+                       (const float*)gate, gate_stride, pairs, heads, dv, eps);
+  else
+    return -1;
+  return (int)hipGetLastError();
+}
+
+static inline unsigned ew_grid(long n) {
+  long g = (n + 255) / 256;
+  return (unsigned)(g < 1 ? 1 : g > 65535 ? 65535 : g);
+}
+
+extern "C" int mx_relu_sq(void* x, int bf16, long n, hipStream_t s) {
+  if (n <= 0) return 0;
+  MX_DISPATCH_T(bf16, hipLaunchKernelGGL((relu_sq_kernel<T>), dim3(ew_grid(n)), dim3(256), 0, s, (T*)x, n));
+  return (int)hipGetLastError();
+}
+
+extern "C" int mx_clamp_swiglu(void* out, const void* gu, int bf16, long gu_stride, long rows, int ff,
+                               float limit, hipStream_t s) {
+  if (rows * ff <= 0) return 0;
+  MX_DISPATCH_T(bf16, hipLaunchKernelGGL((clamp_swiglu_kernel<T>), dim3(ew_grid(rows * ff)), dim3(256), 0,
+                                         s, (T*)out, (const T*)gu, gu_stride, rows, ff, limit));
+  return (int)hipGetLastError();
+}
+
+extern "C" int mx_side_gate(void* out, const void* gpre, const void* table, int bf16, long table_stride,
+                            const int* ids, int col0, long rows, int sd, int vocab, hipStream_t s) {
+  if (rows * sd <= 0) return 0;
+  MX_DISPATCH_T(bf16, hipLaunchKernelGGL((side_gate_kernel<T>), dim3(ew_grid(rows * sd)), dim3(256), 0, s,
+                                         (T*)out, (const T*)gpre, (const T*)table, table_stride, ids, col0,
+                                         rows, sd, vocab));
+  return (int)hipGetLastError();
+}
+
+extern "C" int mx_scale_add_rows(float* out, const void* y, int y_bf16, const int* rows,
+                                 const void* weights, int w_bf16, int sigmoid, long n, int width,
+                                 int out_rows, hipStream_t s) {
+  if (n <= 0) return 0;
+  const dim3 grid((unsigned)n), block(256);
+  if (y_bf16 && w_bf16)
+    hipLaunchKernelGGL((scale_add_rows_kernel<bf16_t, bf16_t>), grid, block, 0, s, out, (const bf16_t*)y,
+                       rows, (const bf16_t*)weights, sigmoid, width, out_rows);
+  else if (y_bf16)
+    hipLaunchKernelGGL((scale_add_rows_kernel<bf16_t, float>), grid, block, 0, s, out, (const bf16_t*)y,
+                       rows, (const float*)weights, sigmoid, width, out_rows);
+  else if (w_bf16)
+    return -1;
+  else
+    hipLaunchKernelGGL((scale_add_rows_kernel<float, float>), grid, block, 0, s, out, (const float*)y,
+                       rows, (const float*)weights, sigmoid, width, out_rows);
+  return (int)hipGetLastError();
+}

@@ -242,6 +242,7 @@ class NulazenModel:
         self.mark_at = None
         self.layer_tap: Optional[list] = None   # tests: fp32 residual after every layer run
         self.invariant = False
+        self._mm_out_dtype = True
         if self.device.type == "cuda":
             # true fp32 / fp32-accumulated products from the vendor library
             torch.backends.cuda.matmul.allow_tf32 = False
@@ -392,8 +393,12 @@ class NulazenModel:
         if h.dtype == torch.float32:
             return F.linear(h, self.head)
         # bf16 operands, fp32 accumulation and fp32 output
-        return torch.mm(h, self.head.t(), out_dtype=torch.float32) if h.is_cuda else \
-            F.linear(h.float(), self.head.float())
+        if h.is_cuda and self._mm_out_dtype:
+            try:
+                return torch.mm(h, self.head.t(), out_dtype=torch.float32)
+            except (TypeError, RuntimeError):
+                self._mm_out_dtype = False   # this build has no fp32-output bf16 product
+        return F.linear(h.float(), self.head.float())
 
 
 # ---------------------------------------------------------------------------------------
