@@ -842,10 +842,14 @@ class LLMEngine:
             for s, n in zip(batch.prefill_seqs, batch.prefill_tokens):
                 base[s.request_id] = r
                 r += n
-            batch.logit_rows = [base[rid] + int(w) for rid, _, want in entries for w in want]
+            wanted = [base[rid] + int(w) for rid, _, want in entries for w in want]
+            # the step gathers ascending, distinct rows; the caller's order is restored here
+            uniq, inverse = np.unique(np.asarray(wanted, dtype=np.int64), return_inverse=True)
+            batch.logit_rows = uniq.tolist()
             self._executing = batch
             logits = self.runner.execute(batch, None, logits_only=True)
             self._executing = None
+            logits = logits[inverse] if len(wanted) else logits
             sched.post_step(batch)
             self.stats["given_steps"] += 1
         for rid in end:

@@ -47,7 +47,7 @@ class ScheduledBatch:
     prefill_start: List[int] = dataclasses.field(default_factory=list)
     prefill_epoch: List[int] = dataclasses.field(default_factory=list)
     # rows of the step (decode rows first, then the prefill chunks in order) whose
-    # logits are wanted, in the order wanted; None: every decode row and the last row
+    # logits are wanted, ascending and distinct; None: every decode row and the last row
     # of each sampled chunk (Scheduler.schedule_given: scoring / replay)
     logit_rows: Optional[List[int]] = None
 

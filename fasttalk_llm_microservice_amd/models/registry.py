@@ -35,9 +35,14 @@ def register(arch: Architecture):
     ARCHITECTURES[arch.name.lower()] = arch
 
 
+_loaded = False
+
+
 def _ensure_loaded():
-    if ARCHITECTURES:
+    global _loaded
+    if _loaded:
         return
+    _loaded = True
     from . import llama_arch, nulazen  # noqa: F401  (each registers itself)
 
 

@@ -1,0 +1,166 @@
+"""Each mechanism of models/mixers.py (and the ops under it) alone against the oracle's
+function for it: one whole sequence, then the same sequence cut in two steps through
+the cache / state the first step left."""
+import torch
+
+import nulazen_oracle as O
+
+from fasttalk_llm_microservice_amd.models import mixers as X
+from fasttalk_llm_microservice_amd.ops import mixers as M
+
+CASES = ["rope", "norms", "latent", "latent_partial_rot", "delta", "delta_gqa_one_tap", "dense", "route",
+         "moe_shared", "moe_top1", "side"]
+EPS = 1e-5
+
+
+def _rand(g, *shape, s=1.0):
+    return (torch.randn(*shape, generator=g) * s).bfloat16().float()
+
+
+def _ctx(T, device, cut=None, page=4, slot=1):
+    """StepContexts of one sequence of T rows: whole, or [0, cut) then [cut, T)."""
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=device)   # noqa: E731
+    nb = (T + page - 1) // page
+    table = list(range(nb - 1, -1, -1))            # pages in reverse order
+    out = []
+    for a, b in ([(0, T)] if cut is None else [(0, cut), (cut, T)]):
+        pos = list(range(a, b))
+        seg = M.Segments(start=i32([0, b - a]), pos0=i32([a]), slot=i32([slot]), kv_len=i32([b]),
+                         block_tables=i32([table]), num=1, max_rows=b - a, max_kv=b)
+        slots = [table[p // page] * page + p % page for p in pos]
+        out.append((a, b, X.StepContext(None, i32(pos), i32(slots), seg)))
+    return out
+
+
+def _tol(dtype):
+    return dict(rtol=3e-4, atol=3e-4) if dtype == torch.float32 else dict(rtol=6e-2, atol=6e-2)
+
+
+def _latent(device, dtype, dims):
+    g = torch.Generator().manual_seed(3)
+    W, T = 40, 29
+    m = {"heads": 3, "dim": 10, "rot_dim": 6, "vdim": 7, "kv_rank": 18, "scale": 0.35,
+         "rot": {"base": 50.0, "dims": dims}}
+    P = {"q": _rand(g, 3 * 16, W, s=0.4), "dkv": _rand(g, 24, W, s=0.3), "dkv.norm": 1 + _rand(g, 18, s=0.1),
+         "uk": _rand(g, 30, 18, s=0.3), "uv": _rand(g, 21, 18, s=0.3), "o": _rand(g, W, 21, s=0.3)}
+    h = _rand(g, T, W)
+    want = O.latent_attention(h, P, "", m, EPS)
+    mix = X.LatentAttention(P.__getitem__, W, 3, 10, 6, 7, 18, 0.35, dims, 50.0, EPS, dtype, device, 64)
+    for cut in (None, 1, 13):
+        cache = torch.zeros(8, 4, 24, dtype=dtype, device=device)
+        got = torch.cat([mix(h[a:b].to(device, dtype), ctx, cache).float().cpu() for a, b, ctx in _ctx(T, device, cut)])
+        torch.testing.assert_close(got, want, **_tol(dtype))
+
+
+def _delta(device, dtype, heads, kvh, dk, dv, taps):
+    g = torch.Generator().manual_seed(4)
+    W, T, lr = 36, 23, 5
+    m = {"heads": heads, "kv_heads": kvh, "dim": dk, "vdim": dv, "conv": taps}
+    P = {"q": _rand(g, kvh * dk, W, s=0.4), "k": _rand(g, kvh * dk, W, s=0.4), "v": _rand(g, heads * dv, W, s=0.4),
+         "q.conv": _rand(g, kvh * dk, taps, s=0.6), "k.conv": _rand(g, kvh * dk, taps, s=0.6),
+         "v.conv": _rand(g, heads * dv, taps, s=0.6), "b": _rand(g, heads, W, s=0.3),
+         "A_log": _rand(g, heads, s=0.5) - 2.0, "norm": 1 + _rand(g, dv, s=0.1), "a1": _rand(g, lr, W, s=0.3),
+         "a2": _rand(g, heads * dk, lr), "dt_bias": _rand(g, heads * dk) - 1.0, "g1": _rand(g, lr, W, s=0.3),
+         "g2": _rand(g, heads * dv, lr), "o": _rand(g, W, heads * dv, s=0.3)}
+    h = _rand(g, T, W)
+    want = O.channel_delta(h, P, "", m, EPS)
+    mix = X.ChannelDelta(P.__getitem__, W, heads, kvh, dk, dv, taps, EPS, dtype, device)
+    for cut in (None, 1, 2, 11):
+        s_shape, c_shape = mix.state_shapes()
+        state = (torch.full((3,) + s_shape, 7.0, device=device), torch.full((3,) + c_shape, 7.0, device=device))
+        got = torch.cat([mix(h[a:b].to(device, dtype), ctx, state).float().cpu() for a, b, ctx in _ctx(T, device, cut)])
+        torch.testing.assert_close(got, want, **_tol(dtype))
+        assert float(state[0][0].min()) == 7.0 and float(state[0][2].max()) == 7.0   # other slots untouched
+
+
+def _moe(device, dtype, E, top, groups, shared):
+    g = torch.Generator().manual_seed(5)
+    W, T, ff = 32, 41, 12
+    P = {"router": _rand(g, E, W, s=0.5), "correction": _rand(g, E, s=0.3) - 0.2}
+    for e in range(E):
+        P.update({f"e{e}.gate": _rand(g, ff, W, s=0.5), f"e{e}.up": _rand(g, ff, W, s=0.5),
+                  f"e{e}.down": _rand(g, W, ff, s=0.4)})
+    m = {"expert": {"ff": ff, "limit": 1.1}, "router": {"experts": E, "top": top}}
+    if groups:
+        m["router"]["groups"] = {"count": groups[0], "keep": groups[1]}
+    if shared:
+        m["shared"] = {"ff": 20, "limit": 0.8}
+        P.update({"shared.gate": _rand(g, 20, W, s=0.5), "shared.up": _rand(g, 20, W, s=0.5),
+                  "shared.down": _rand(g, W, 20, s=0.4), "shared.sg": _rand(g, 1, W, s=0.5)})
+    h = _rand(g, T, W)
+    want = O.moe_ff(h, P, "", m)
+    ff_ = X.MoEFF(P.__getitem__, E, top, 1.1, groups[0] if groups else 1, groups[1] if groups else 1,
+                  0.8 if shared else None, dtype, device)
+    got = ff_(h.to(device, dtype)).float().cpu()
+    if dtype == torch.float32:
+        torch.testing.assert_close(got, want, **_tol(dtype))
+    else:   # a rounded router input may flip a close choice for a few tokens
+        bad = ((got - want).abs().amax(-1) > 0.1).float().mean()
+        assert bad <= 0.1
+
+
+def run(case, device, dtype):
+    g = torch.Generator().manual_seed(1)
+    if case == "rope":
+        tab = M.rope_table(40, 6, 37.0)
+        x = _rand(g, 40, 2, 9)
+        want = O.rotate(x, 6, 37.0)
+        half = 3
+        got = x.clone()
+        got[..., :half] = x[..., :half] * tab[:, None, :half] - x[..., half:6] * tab[:, None, half:]
+        got[..., half:6] = x[..., half:6] * tab[:, None, :half] + x[..., :half] * tab[:, None, half:]
+        torch.testing.assert_close(got, want, rtol=1e-6, atol=1e-6)
+    elif case == "norms":
+        x, y = _rand(g, 5, 50), _rand(g, 5, 50)
+        w1, w2, vec = 1 + _rand(g, 50, s=0.1), 1 + _rand(g, 50, s=0.1), _rand(g, 50)
+        xd = x.clone().to(device)
+        out, cast = M.add_rms_norm_rows(xd, y.to(device, dtype), w1.to(device), EPS, vec.to(device),
+                                        w2.to(device), dtype, True)
+        want_x = x + O.rms(y, EPS, w1) + vec
+        torch.testing.assert_close(xd.cpu(), want_x, rtol=1e-5, atol=1e-5)
+        torch.testing.assert_close(out.float().cpu(), O.rms(want_x, EPS, w2), **_tol(dtype))
+        torch.testing.assert_close(cast.float().cpu(), want_x, **_tol(dtype))
+    elif case == "latent":
+        _latent(device, dtype, 6)
+    elif case == "latent_partial_rot":
+        _latent(device, dtype, 2)
+    elif case == "delta":
+        _delta(device, dtype, 4, 2, 9, 11, 4)
+    elif case == "delta_gqa_one_tap":
+        _delta(device, dtype, 3, 1, 16, 5, 1)
+    elif case == "dense":
+        P = {"up": _rand(g, 30, 20, s=0.4), "down": _rand(g, 20, 30, s=0.4)}
+        h = _rand(g, 9, 20)
+        got = X.DenseFF(P.__getitem__, dtype, device)(h.to(device, dtype)).float().cpu()
+        torch.testing.assert_close(got, O.dense_ff(h, P, ""), **_tol(dtype))
+    elif case == "route":
+        for E, top, grp in ((8, 3, (4, 2)), (9, 2, (3, 1)), (7, 7, None), (10, 1, (5, 4))):
+            P = {"router": _rand(g, E, 16, s=0.7), "correction": _rand(g, E, s=0.4) - 0.3}
+            h = _rand(g, 50, 16)
+            r = {"experts": E, "top": top}
+            if grp:
+                r["groups"] = {"count": grp[0], "keep": grp[1]}
+            want = O.route(h, P, "", r)
+            z = (h @ P["router"].T).to(device)
+            idx, wts = M.moe_topk(z, P["correction"].to(device), top, grp[0] if grp else 1, grp[1] if grp else 1)
+            for t, (ids, ws) in enumerate(want):
+                assert sorted(idx[t].tolist()) == sorted(ids)
+                torch.testing.assert_close(wts[t].cpu().sort().values, torch.stack(ws).sort().values,
+                                           rtol=1e-5, atol=1e-7)
+    elif case == "moe_shared":
+        _moe(device, dtype, 8, 3, (4, 2), True)
+    elif case == "moe_top1":
+        _moe(device, dtype, 5, 1, None, False)
+    elif case == "side":
+        W, sd, V = 24, 4, 30
+        P = {"gate": _rand(g, sd, W, s=0.5), "proj": _rand(g, W, sd, s=0.5), "norm": 1 + _rand(g, W, s=0.1)}
+        table = _rand(g, V, 3 * sd)
+        ids = torch.randint(0, V, (11,), generator=g)
+        x = _rand(g, 11, W)
+        side = X.TokenSide(P.__getitem__, table.to(device, dtype), sd, sd, dtype, device)
+        ctx = X.StepContext(ids.int().to(device), None, None, None)
+        got = side(x.to(device, dtype), ctx).float().cpu()
+        want = (O.gelu_tanh(x @ P["gate"].T) * table[ids][:, sd:2 * sd]) @ P["proj"].T
+        torch.testing.assert_close(got, want, **_tol(dtype))
+    else:
+        raise KeyError(case)
