@@ -178,7 +178,23 @@ def main():
     ap.add_argument("--agent-tools", type=float, default=-1.0, metavar="FRAC",
                     help="BASELINE config 5: agent with JSON-guided tool calls, FRAC of the turns "
                          "ask for a web search (stub backend); e.g. 0.2")
+    ap.add_argument("--engine-compare", default="", metavar="MODELS",
+                    help="instead of the headline benchmark: engine-level prefill / decode throughput "
+                         "of these registry models side by side (comma separated, random weights), "
+                         "e.g. nulazen-2k,llama-2k-4l (bench/engine_compare.py)")
+    ap.add_argument("--compare-prompts", default="512,2048,4096")
+    ap.add_argument("--compare-batches", default="1,8,32")
+    ap.add_argument("--compare-dtype", default="bfloat16", choices=["bfloat16", "float32"])
     a = ap.parse_args()
+    if a.engine_compare:
+        sys.path.insert(0, os.path.join(ROOT, "bench"))
+        import engine_compare
+
+        engine_compare.main([m for m in a.engine_compare.split(",") if m],
+                            [int(x) for x in a.compare_prompts.split(",")],
+                            [int(x) for x in a.compare_batches.split(",")], gen=a.gen if a.gen != 128 else 64,
+                            dtype=a.compare_dtype)
+        return
     if "WORLD_SIZE" not in os.environ:
         if (a.gpus or 1) > 1:
             sys.exit(_launch_ranks(a.gpus, sys.argv[1:]))

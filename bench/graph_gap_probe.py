@@ -66,7 +66,7 @@ def main():
     nb = r._bucket(len(seqs))
     g = r.graphs[nb]
     st = r.stg[0]
-    nw = 10 * r.max_decode_batch + nb * r.max_blocks_per_seq
+    nw = 12 * r.max_decode_batch + nb * r.max_blocks_per_seq
 
     def timed(body):
         body()

@@ -43,7 +43,12 @@ int mx_latent_max_rank();
 int mx_latent_attention(float* out, const float* qa, const float* qr, const void* cache, int cache_bf16,
                         const int* start, const int* pos0, const int* kv_len, const int* bt, int bt_stride,
                         int num_segs, int max_rows, int heads, long total_rows, int rank, int dr,
-                        int block_size, int num_blocks, float scale, hipStream_t s);
+                        int block_size, int num_blocks, float scale, int skip_from, hipStream_t s);
+int mx_causal_softmax(void* P, int p_bf16, const float* S, long rows, int rows_per_head, int first_pos, int ncols,
+                      float scale, hipStream_t s);
+int mx_moe_pairs(float* out, void* y, const void* h, int bf16, long h_stride, const int* idx, const float* wts,
+                 const void* wgu, const void* wdown, long rows, int top, int experts, int ff, int width,
+                 float limit, hipStream_t s);
 int mx_moe_topk(int* idx, float* wts, const float* z, const float* corr, long rows, int experts, int top,
                 int groups, int keep, hipStream_t s);
 }
@@ -262,7 +267,7 @@ void latent_q_rope(Tensor qn, Tensor qr, Tensor q, Tensor table, int64_t dims, T
 }
 
 void latent_attention(Tensor out, Tensor qa, Tensor qr, Tensor cache, Tensor start, Tensor pos0, Tensor kv_len,
-                      Tensor bt, int64_t num_segs, int64_t max_rows, double scale, int64_t rank) {
+                      Tensor bt, int64_t num_segs, int64_t max_rows, double scale, int64_t rank, int64_t skip_from) {
   check_f32(out, "out");
   check_f32(qa, "qa");
   check_f32(qr, "qr");
@@ -277,8 +282,17 @@ void latent_attention(Tensor out, Tensor qa, Tensor qr, Tensor cache, Tensor sta
   chk(mx_latent_attention(out.data_ptr<float>(), qa.data_ptr<float>(), qr.data_ptr<float>(), cache.data_ptr(),
                           bf(cache), start.data_ptr<int>(), pos0.data_ptr<int>(), kv_len.data_ptr<int>(),
                           bt.data_ptr<int>(), (int)bt.size(1), (int)num_segs, (int)max_rows, (int)heads, t,
-                          (int)rank, (int)dr, (int)cache.size(1), (int)cache.size(0), (float)scale, stream()),
+                          (int)rank, (int)dr, (int)cache.size(1), (int)cache.size(0), (float)scale, (int)skip_from,
+                          stream()),
       "latent_attention");
+}
+
+void causal_softmax(Tensor P, Tensor S, int64_t rows_per_head, int64_t first_pos, double scale) {
+  check_f32(S, "S");
+  TORCH_CHECK(S.dim() == 2 && P.is_cuda() && is_act(P) && P.is_contiguous() && P.sizes() == S.sizes() &&
+              rows_per_head >= 1 && S.size(0) % rows_per_head == 0 && first_pos >= 0, "causal_softmax shapes");
+  chk(mx_causal_softmax(P.data_ptr(), bf(P), S.data_ptr<float>(), S.size(0), (int)rows_per_head, (int)first_pos,
+                        (int)S.size(1), (float)scale, stream()), "causal_softmax");
 }
 
 void moe_topk(Tensor idx, Tensor wts, Tensor z, Tensor corr, int64_t top, int64_t groups, int64_t keep) {
@@ -290,6 +304,27 @@ void moe_topk(Tensor idx, Tensor wts, Tensor z, Tensor corr, int64_t top, int64_
               wts.numel() == z.size(0) * top, "moe_topk shapes");
   chk(mx_moe_topk(idx.data_ptr<int>(), wts.data_ptr<float>(), z.data_ptr<float>(), corr.data_ptr<float>(),
                   z.size(0), (int)z.size(1), (int)top, (int)groups, (int)keep, stream()), "moe_topk");
+}
+
+void moe_pairs(Tensor out, Tensor h, Tensor idx, Tensor wts, Tensor wgu, Tensor wdown, double limit) {
+  check_f32(out, "out");
+  check_rows(h, "h");
+  check_i32(idx, "idx");
+  check_f32(wts, "wts");
+  TORCH_CHECK(wgu.is_cuda() && wgu.is_contiguous() && wgu.dim() == 3 && wdown.is_cuda() && wdown.is_contiguous() &&
+              wdown.dim() == 3 && wgu.scalar_type() == h.scalar_type() && wdown.scalar_type() == h.scalar_type(),
+              "expert weights");
+  const int64_t rows = h.size(0), width = h.size(1), experts = wgu.size(0), ff = wgu.size(1) / 2;
+  TORCH_CHECK(idx.dim() == 2 && idx.size(0) == rows && wts.sizes() == idx.sizes(), "idx / wts");
+  const int64_t top = idx.size(1);
+  TORCH_CHECK(wgu.size(2) == width && wdown.size(0) == experts && wdown.size(1) == width && wdown.size(2) == ff &&
+              wgu.size(1) == 2 * ff && out.dim() == 2 && out.size(0) == rows && out.size(1) == width,
+              "moe_pairs shapes");
+  TORCH_CHECK(((uintptr_t)h.data_ptr()) % 16 == 0, "h alignment");
+  Tensor y = at::empty({rows * top, ff}, h.options());
+  chk(mx_moe_pairs(out.data_ptr<float>(), y.data_ptr(), h.data_ptr(), bf(h), h.stride(0), idx.data_ptr<int>(),
+                   wts.data_ptr<float>(), wgu.data_ptr(), wdown.data_ptr(), rows, (int)top, (int)experts, (int)ff,
+                   (int)width, (float)limit, stream()), "moe_pairs");
 }
 
 }  // namespace
@@ -307,7 +342,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("latent_kv_write", &latent_kv_write);
   m.def("latent_q_rope", &latent_q_rope);
   m.def("latent_attention", &latent_attention);
+  m.def("causal_softmax", &causal_softmax);
   m.def("moe_topk", &moe_topk);
+  m.def("moe_pairs", &moe_pairs);
   m.def("delta_max_dk", []() { return (int64_t)mx_delta_max_dk(); });
   m.def("latent_max_rank", []() { return (int64_t)mx_latent_max_rank(); });
 }

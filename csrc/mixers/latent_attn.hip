@@ -80,12 +80,12 @@ latent_attention_kernel(float* __restrict__ out, const float* __restrict__ qa, c
                         const TC* __restrict__ cache, const int* __restrict__ start,
                         const int* __restrict__ pos0, const int* __restrict__ kv_len,
                         const int* __restrict__ bt, int bt_stride, int heads, long total_rows, int rank,
-                        int dr, int block_size, int num_blocks, float scale) {
+                        int dr, int block_size, int num_blocks, float scale, int skip_from) {
   extern __shared__ float smem[];
   const int s = blockIdx.y;
   const int r0 = start[s], n = start[s + 1] - r0;
   const int rel = blockIdx.x;
-  if (rel >= n) return;
+  if (rel >= n || (skip_from > 0 && n >= skip_from)) return;   // long segments: the product path
   const long row = r0 + rel;
   const int wid = threadIdx.x >> 6, lane = threadIdx.x & 63, nw = blockDim.x >> 6;
   const int width = rank + dr;
@@ -147,9 +147,51 @@ latent_attention_kernel(float* __restrict__ out, const float* __restrict__ qa, c
   }
 }
 
+// P[r, j] = softmax_j(scale * S[r, j]) over the keys j <= first_pos + (r mod rows_per_head),
+// 0 beyond (rows r = head * rows_per_head + query row); fp32 statistics, P in TP
+template <typename TP, int NT>
+__global__ void causal_softmax_kernel(TP* __restrict__ P, const float* __restrict__ S, int rows_per_head,
+                                      int first_pos, int ncols, float scale) {
+  __shared__ float red[NT / 64];
+  __shared__ float bmax;
+  const long r = blockIdx.x;
+  const int valid = min(first_pos + (int)(r % rows_per_head) + 1, ncols);
+  const float* sr = S + r * ncols;
+  float m = -INFINITY;
+  for (int j = threadIdx.x; j < valid; j += NT) m = fmaxf(m, sr[j] * scale);
+  m = ft::wave_max(m);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float b = red[0];
+    for (int w = 1; w < NT / 64; ++w) b = fmaxf(b, red[w]);
+    bmax = b;
+  }
+  __syncthreads();
+  m = bmax;
+  float sum = 0.f;
+  for (int j = threadIdx.x; j < valid; j += NT) sum += expf(sr[j] * scale - m);
+  sum = block_sum<NT>(sum, red);
+  const float inv = sum > 0.f ? 1.0f / sum : 0.f;
+  for (int j = threadIdx.x; j < ncols; j += NT)
+    st(P, r * ncols + j, j < valid ? expf(sr[j] * scale - m) * inv : 0.f);
+}
+
 }  // namespace mx
 
 using namespace mx;
+
+extern "C" int mx_causal_softmax(void* P, int p_bf16, const float* S, long rows, int rows_per_head,
+                                 int first_pos, int ncols, float scale, hipStream_t s) {
+  if (rows <= 0 || ncols <= 0) return 0;
+  if (p_bf16)
+    hipLaunchKernelGGL((causal_softmax_kernel<bf16_t, 256>), dim3((unsigned)rows), dim3(256), 0, s, (bf16_t*)P, S,
+                       rows_per_head, first_pos, ncols, scale);
+  else
+    hipLaunchKernelGGL((causal_softmax_kernel<float, 256>), dim3((unsigned)rows), dim3(256), 0, s, (float*)P, S,
+                       rows_per_head, first_pos, ncols, scale);
+  return (int)hipGetLastError();
+}
 
 extern "C" int mx_latent_kv_write(const void* dkv, int bf16, long stride, const float* w, float eps,
                                   const float* table, int table_rows, int dims, const int* positions,
@@ -186,31 +228,33 @@ template <typename TC, int RPL>
 static void launch_latent(dim3 grid, size_t lds, hipStream_t s, float* out, const float* qa, const float* qr,
                           const void* cache, const int* start, const int* pos0, const int* kv_len,
                           const int* bt, int bt_stride, int heads, long total_rows, int rank, int dr,
-                          int block_size, int num_blocks, float scale) {
+                          int block_size, int num_blocks, float scale, int skip_from) {
   hipLaunchKernelGGL((latent_attention_kernel<TC, RPL>), grid, dim3(256), lds, s, out, qa, qr,
                      (const TC*)cache, start, pos0, kv_len, bt, bt_stride, heads, total_rows, rank, dr,
-                     block_size, num_blocks, scale);
+                     block_size, num_blocks, scale, skip_from);
 }
 
 extern "C" int mx_latent_attention(float* out, const float* qa, const float* qr, const void* cache,
                                    int cache_bf16, const int* start, const int* pos0, const int* kv_len,
                                    const int* bt, int bt_stride, int num_segs, int max_rows, int heads,
                                    long total_rows, int rank, int dr, int block_size, int num_blocks,
-                                   float scale, hipStream_t s) {
+                                   float scale, int skip_from, hipStream_t s) {
   if (num_segs <= 0 || max_rows <= 0) return 0;
   if (rank < 1 || rank > mx_latent_max_rank() || max_rows > 65535 * 32 || num_segs > 65535) return -1;
   const size_t lds = (size_t)4 * (rank + dr) * sizeof(float);
   if (lds > 60 * 1024) return -2;
+  if (skip_from > 0 && max_rows >= skip_from) max_rows = skip_from - 1;
+  if (max_rows <= 0) return 0;
   const dim3 grid(max_rows, num_segs);
   const int need = (rank + 63) / 64;
 #define MX_LAT(RPL)                                                                                     \
   do {                                                                                                  \
     if (cache_bf16)                                                                                     \
       launch_latent<bf16_t, RPL>(grid, lds, s, out, qa, qr, cache, start, pos0, kv_len, bt, bt_stride,  \
-                                 heads, total_rows, rank, dr, block_size, num_blocks, scale);           \
+                                 heads, total_rows, rank, dr, block_size, num_blocks, scale, skip_from); \
     else                                                                                                \
       launch_latent<float, RPL>(grid, lds, s, out, qa, qr, cache, start, pos0, kv_len, bt, bt_stride,   \
-                                heads, total_rows, rank, dr, block_size, num_blocks, scale);            \
+                                heads, total_rows, rank, dr, block_size, num_blocks, scale, skip_from); \
   } while (0)
   if (need <= 1) MX_LAT(1);
   else if (need <= 2) MX_LAT(2);

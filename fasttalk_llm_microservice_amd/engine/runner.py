@@ -59,15 +59,19 @@ def _pow2_ceil(x: int) -> int:
     return 1 << max(0, (x - 1).bit_length())
 
 
+# int32 words per row ahead of the block tables: 8 small fields (7 used), 2 f32, 1 int64 seed
+IN_HEAD = 12
+
+
 def input_words(mb: int, max_blocks: int) -> int:
-    return 10 * mb + mb * max_blocks
+    return IN_HEAD * mb + mb * max_blocks
 
 
 def _input_views(buf: torch.Tensor, mb: int, max_blocks: int):
-    """(small int32 [6mb], f32 [2mb], seeds int64 [mb], block tables int32 [mb, max_blocks])
+    """(small int32 [8mb], f32 [2mb], seeds int64 [mb], block tables int32 [mb, max_blocks])
     views of one int32 buffer of input_words() elements."""
-    return (buf[0:6 * mb], buf[6 * mb:8 * mb].view(torch.float32), buf[8 * mb:10 * mb].view(torch.int64),
-            buf[10 * mb:].view(mb, max_blocks))
+    return (buf[0:8 * mb], buf[8 * mb:10 * mb].view(torch.float32), buf[10 * mb:12 * mb].view(torch.int64),
+            buf[12 * mb:].view(mb, max_blocks))
 
 
 class _Uploader:
@@ -130,7 +134,7 @@ class _Uploader:
 
 class _Staging:
     """Pinned host mirror of the decode graph's device inputs + its output copy.
-    int32 ``small`` fields: ids | pos | slots | seq_lens | top_k | steps."""
+    int32 ``small`` fields: ids | pos | slots | seq_lens | top_k | steps | state slots."""
 
     def __init__(self, mb: int, max_blocks: int, pin: bool, gpu: bool):
         i32 = torch.int32
@@ -284,6 +288,11 @@ class ModelRunner:
         self.d_seq_lens = self.d_small[3 * mb:4 * mb]
         self.d_top_k = self.d_small[4 * mb:5 * mb]
         self.d_steps = self.d_small[5 * mb:6 * mb]
+        self.d_sslots = self.d_small[6 * mb:7 * mb]      # recurrent-state slots (stateful models)
+        self.d_rowstart = torch.arange(mb + 1, dtype=i32, device=dv)   # one-row segments
+        # decode graphs of models that bound their captured steps' rows (Nulazen: the
+        # per-pair expert kernels)
+        self.max_graph_rows = int(getattr(self.model, "max_graph_rows", 1 << 30))
         self.d_temp = self.d_f32[0:mb]
         self.d_top_p = self.d_f32[mb:2 * mb]
         self.d_out = torch.zeros(mb, dtype=i32, device=dv)
@@ -476,7 +485,7 @@ class ModelRunner:
     def _bucket(self, b: int) -> Optional[int]:
         for s in self.graph_sizes:
             if s >= b:
-                return s
+                return s if s <= self.max_graph_rows else None
         return None
 
     # ------------------------------------------------------------------ execution
@@ -705,7 +714,8 @@ class ModelRunner:
 
         return Segments(start=d["sg_start"], pos0=d["sg_pos0"], slot=d["sg_slot"], kv_len=d["sg_len"],
                         block_tables=d["sg_bt"], num=host["num_segs"], max_rows=host["max_rows"],
-                        max_kv=host["max_kv"])
+                        max_kv=host["max_kv"],
+                        host=(host["sg_start"].tolist(), host["sg_pos0"].tolist(), host["sg_len"].tolist()))
 
     def _wait(self, ev=None):
         """Block until the GPU work queued so far (or up to ``ev``) is done WITHOUT
@@ -1102,6 +1112,11 @@ class ModelRunner:
             nbk = len(s.block_ids)
             bt[i, :nbk] = s.block_ids
             maxblk = max(maxblk, nbk)
+        if self.stateful:
+            ss = hs[6 * mb:7 * mb]
+            for i, s in enumerate(seqs):
+                ss[i] = s.state_slot
+            ss[n:nb] = -1   # padding rows touch no state
         temp, topp, topk, seeds, steps = self._sampling_arrays(seqs)
         hs[4 * mb:4 * mb + n] = topk
         hs[5 * mb:5 * mb + n] = steps
@@ -1167,7 +1182,7 @@ class ModelRunner:
 
     def _decode_enqueue(self, st: "_Staging", nb: int, n: int, from_device: bool = False,
                         gather: Optional[np.ndarray] = None, fwd_only: bool = False):
-        nw = 10 * self.max_decode_batch + nb * self.max_blocks_per_seq
+        nw = IN_HEAD * self.max_decode_batch + nb * self.max_blocks_per_seq
         if self._gaps is not None:   # g: a split step, closed by its sampler (sample_launch)
             self._gap_mark(True, "g" if fwd_only else "d")
         self.d_in[:nw].copy_(st.h_in[:nw], non_blocking=True)
@@ -1257,10 +1272,17 @@ class ModelRunner:
 
     def _decode_meta(self, nb: int) -> AttnMeta:
         assert nb <= self.max_decode_rows
-        return AttnMeta(positions=self.d_positions[:nb], slot_mapping=self.d_slots[:nb],
+        meta = AttnMeta(positions=self.d_positions[:nb], slot_mapping=self.d_slots[:nb],
                         logits_indices=self.d_logits_idx[:nb], num_decode=nb,
                         dec_block_tables=self.d_bt[:nb], dec_seq_lens=self.d_seq_lens[:nb],
                         tmp_out=self.tmp_out, tmp_ml=self.tmp_ml, dec_counters=self.dec_counters)
+        if self.stateful:   # every decode row is a one-row segment of its sequence
+            from ..ops.mixers import Segments
+
+            meta.segments = Segments(start=self.d_rowstart[:nb + 1], pos0=self.d_positions[:nb],
+                                     slot=self.d_sslots[:nb], kv_len=self.d_seq_lens[:nb],
+                                     block_tables=self.d_bt[:nb], num=nb, max_rows=1)
+        return meta
 
     def _graph_body(self, nb: int, keep: bool = False):
         meta = self._decode_meta(nb)
@@ -1283,9 +1305,10 @@ class ModelRunner:
         graph; the logits stay allocated."""
         self._assert_no_pending_split("split-graph capture")
         t0 = time.time()
-        saved = (self.d_slots[:nb].clone(), self.d_seq_lens[:nb].clone())
+        saved = (self.d_slots[:nb].clone(), self.d_seq_lens[:nb].clone(), self.d_sslots[:nb].clone())
         self.d_slots[:nb].fill_(-1)
         self.d_seq_lens[:nb].fill_(0)
+        self.d_sslots[:nb].fill_(-1)
 
         def fwd():
             h = self.model.forward(self.d_input_ids[:nb], self._decode_meta(nb), self.kv)
@@ -1312,6 +1335,7 @@ class ModelRunner:
             samp(lg)
         self.d_slots[:nb].copy_(saved[0])
         self.d_seq_lens[:nb].copy_(saved[1])
+        self.d_sslots[:nb].copy_(saved[2])
         self.graphs_split[nb] = (gf, gs)
         self.stats["captures"] += 1
         log.info("captured split decode graphs batch=%d in %.2fs", nb, time.time() - t0)
@@ -1325,10 +1349,12 @@ class ModelRunner:
         first capture and must be of the same kind for every later one."""
         self._assert_no_pending_split("graph capture")
         t0 = time.time()
-        # inputs must be valid for the warm-up/capture run: no KV writes, empty contexts
-        saved = (self.d_slots[:nb].clone(), self.d_seq_lens[:nb].clone())
+        # inputs must be valid for the warm-up/capture run: no KV writes, empty contexts,
+        # no recurrent-state slot touched
+        saved = (self.d_slots[:nb].clone(), self.d_seq_lens[:nb].clone(), self.d_sslots[:nb].clone())
         self.d_slots[:nb].fill_(-1)
         self.d_seq_lens[:nb].fill_(0)
+        self.d_sslots[:nb].fill_(-1)
         s = torch.cuda.Stream(self.device)
         s.wait_stream(torch.cuda.current_stream(self.device))
         with torch.cuda.stream(s), self._long_waits():
@@ -1341,6 +1367,7 @@ class ModelRunner:
             self._graph_body(nb, keep=True)
         self.d_slots[:nb].copy_(saved[0])
         self.d_seq_lens[:nb].copy_(saved[1])
+        self.d_sslots[:nb].copy_(saved[2])
         self.graphs[nb] = g
         self.stats["captures"] += 1
         log.info("captured decode graph batch=%d in %.2fs", nb, time.time() - t0)

@@ -73,6 +73,10 @@ MODELS = {
     # serving shape, a fraction of the weights)
     "llama3-8b-2l": ModelConfig("llama3-8b-2l", 4096, 2, 32, 8, 128, 14336),
     "llama3-70b-2l": ModelConfig("llama3-70b-2l", 8192, 2, 64, 8, 128, 28672),
+    # 4-layer stacks at 2048 / 4096 width, 32k vocabulary (engine-level comparisons with
+    # other architectures at equal width and depth: bench.py --engine-compare)
+    "llama-2k-4l": ModelConfig("llama-2k-4l", 2048, 4, 16, 4, 128, 8192, vocab_size=32768),
+    "llama-4k-4l": ModelConfig("llama-4k-4l", 4096, 4, 32, 8, 128, 14336, vocab_size=32768),
     # small shapes for CPU tests (keep kernel constraints: hidden % 512 == 0)
     "tiny": ModelConfig("tiny", 512, 2, 8, 2, 64, 1024, vocab_size=128256),
     "tiny-gqa4": ModelConfig("tiny-gqa4", 512, 2, 8, 2, 64, 1536, vocab_size=128256),

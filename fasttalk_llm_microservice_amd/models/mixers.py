@@ -58,6 +58,10 @@ class LatentAttention:
         self.wo = get("o").to(device, dtype).contiguous()
         self.table = M.rope_table(max_pos, rot_dims, rot_base, device=device)
 
+    # segments of this many rows or more run as matrix products (ops.mixers
+    # latent_attention_products), shorter ones and decode rows in the per-row kernel
+    PRODUCT_ROWS = 32
+
     def cache_width(self) -> int:
         return self.rank + self.dr
 
@@ -70,7 +74,17 @@ class LatentAttention:
         qn, qr = M.latent_q_rope(q, self.table, self.rot_dims, ctx.positions, self.heads, self.dn,
                                  self.dr)
         qa = torch.bmm(qn.transpose(0, 1), self.wuk)                 # [heads, T, rank]
-        ol = M.latent_attention(qa, qr, cache, ctx.seg, self.scale, self.rank)
+        seg = ctx.seg
+        if seg.host is not None and seg.max_rows >= self.PRODUCT_ROWS:
+            # prefill chunks: two tiled products per segment; short segments and decode
+            # rows (if any) keep the per-row kernel
+            ol = torch.zeros_like(qa)
+            M.latent_attention(qa, qr, cache, seg, self.scale, self.rank, skip_from=self.PRODUCT_ROWS,
+                               out=ol)
+            M.latent_attention_products(ol, qa, qr, cache, seg, self.scale, self.rank,
+                                        self.PRODUCT_ROWS, self.dtype)
+        else:
+            ol = M.latent_attention(qa, qr, cache, seg, self.scale, self.rank)
         o = torch.bmm(ol, self.wuvT)                                  # [heads, T, vdim]
         o = o.transpose(0, 1).reshape(t, self.heads * self.dv).to(self.dtype)
         return F.linear(o, self.wo)
@@ -166,6 +180,10 @@ class MoEFF:
         out = torch.zeros(t, width, dtype=torch.float32, device=h.device)
         z = F.linear(h.float(), self.router)
         idx, wts = M.moe_topk(z, self.correction, self.top, self.groups, self.keep)
+        if t <= self.PAIR_ROWS:
+            # decode-size steps: per-pair weight streaming, nothing read back on the host
+            M.moe_pairs(out, h, idx, wts, self.wgu, self.wdown, self.limit)
+            return self._shared(out, h)
         flat = idx.view(-1).long()
         order = torch.argsort(flat, stable=True)
         counts = torch.bincount(flat, minlength=self.e).tolist()
@@ -179,6 +197,13 @@ class MoEFF:
             y = M.clamp_swiglu(F.linear(hs[a:a + n], self.wgu[e]), self.limit)
             M.scale_add_rows(out, F.linear(y, self.wdown[e]), rows[a:a + n], w[a:a + n])
             a += n
+        return self._shared(out, h)
+
+    # rows up to which every (row, expert) pair streams its expert's weights (decode);
+    # above, rows are sorted by expert and each expert runs one tiled product
+    PAIR_ROWS = 64
+
+    def _shared(self, out, h):
         if self.shared is not None:
             wgu, wdown = self.shared
             gu = F.linear(h, wgu)

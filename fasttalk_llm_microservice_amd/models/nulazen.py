@@ -225,7 +225,10 @@ class NulazenCache:
 
 class NulazenModel:
     needs_state_slots = True     # the runner hands every sequence a state slot
-    supports_graphs = False      # expert dispatch reads its group sizes on the host
+    # decode steps up to this many rows run without a host round trip (per-pair expert
+    # kernels) and are captured in hipGraphs; larger steps sort rows by expert on the host
+    supports_graphs = True
+    max_graph_rows = MoEFF.PAIR_ROWS
 
     def __init__(self, cfg: NulazenConfig, device, dtype=torch.bfloat16, comm: TPComm = SINGLE,
                  max_model_len: int = 8192, quantization: Optional[str] = None):
@@ -442,6 +445,13 @@ PRESETS = {
         {"type": DELTA, "mixer": _delta(16, 128, 128), "mlp": _moe(32, 4, 1024, 2048, groups=4, keep=2)},
         {"type": DELTA, "mixer": _delta(16, 128, 128), "mlp": _moe(32, 4, 1024, 2048, groups=4, keep=2)},
         {"type": LATENT, "mixer": _latent(16, 128, 64, 128, 512), "mlp": _moe(32, 4, 1024, 2048, groups=4, keep=2)},
+    ], side=64),
+    # the same stack at 4096 width
+    "nulazen-4k": _preset("nulazen-4k", 32768, 4096, [
+        {"type": DELTA, "mixer": _delta(32, 128, 128), "mlp": {"kind": "dense", "ff": 14336}},
+        {"type": DELTA, "mixer": _delta(32, 128, 128), "mlp": _moe(64, 6, 1408, 2816, groups=8, keep=4)},
+        {"type": DELTA, "mixer": _delta(32, 128, 128), "mlp": _moe(64, 6, 1408, 2816, groups=8, keep=4)},
+        {"type": LATENT, "mixer": _latent(32, 128, 64, 128, 512), "mlp": _moe(64, 6, 1408, 2816, groups=8, keep=4)},
     ], side=64),
 }
 

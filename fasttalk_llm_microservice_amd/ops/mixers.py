@@ -61,6 +61,8 @@ class Segments:
     num: int
     max_rows: int                # longest segment (rows)
     max_kv: int = 0              # longest context (tokens); 0 = unknown
+    # host copies of start / pos0 / kv_len (eager steps; None inside captured graphs)
+    host: Optional[tuple] = None
 
 
 # ---------------------------------------------------------------------------------
@@ -176,18 +178,88 @@ def latent_q_rope(q, table, rot_dims: int, positions, heads: int, dn: int, dr: i
     return ref.latent_q_rope(q, table, rot_dims, positions, heads, dn, dr)
 
 
-def latent_attention(qa, qr, cache, seg: Segments, scale: float, rank: int) -> torch.Tensor:
+def latent_attention(qa, qr, cache, seg: Segments, scale: float, rank: int,
+                     skip_from: int = 0, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Causal softmax attention over the paged latent cache.  ``qa`` fp32 [heads, T,
     rank]: the unrotated query parts carried into latent space (q W_uk); ``qr`` fp32
     [T, heads, dr]: the rotated parts.  Score = (qa . c + qr . k_rot) * scale; all heads
     share the cached row, whose first ``rank`` entries are also the value.  Returns
-    fp32 [heads, T, rank]."""
+    fp32 [heads, T, rank].  ``skip_from`` > 0: segments of that many rows or more are
+    left to the caller (:func:`latent_attention_products`)."""
     if qa.is_cuda:
-        out = torch.empty_like(qa)
+        if out is None:
+            out = torch.empty_like(qa)
         native_mixers().latent_attention(out, qa, qr, cache, seg.start, seg.pos0, seg.kv_len,
-                                         seg.block_tables, seg.num, seg.max_rows, scale, rank)
+                                         seg.block_tables, seg.num, seg.max_rows, scale, rank,
+                                         skip_from)
         return out
-    return ref.latent_attention(qa, qr, cache, seg, scale, rank)
+    r = ref.latent_attention(qa, qr, cache, seg, scale, rank)
+    if out is not None:
+        out.copy_(r)
+        return out
+    return r
+
+
+def causal_softmax(s, rows_per_head: int, first_pos: int, scale: float, out_dtype):
+    """P = softmax(scale * S) per row over the keys j <= first_pos + (row mod
+    rows_per_head), zeros beyond; S fp32 [heads * rows_per_head, keys]."""
+    if s.is_cuda:
+        p = torch.empty(s.shape, dtype=out_dtype, device=s.device)
+        native_mixers().causal_softmax(p, s, rows_per_head, first_pos, scale)
+        return p
+    return ref.causal_softmax(s, rows_per_head, first_pos, scale, out_dtype)
+
+
+_MM_F32_OUT = {}
+
+
+def mm_f32(a, b):
+    """a @ b with fp32 accumulation and fp32 output (operands fp32, or bf16 where the
+    vendor library returns fp32 from bf16 operands; otherwise widened first)."""
+    if a.dtype == torch.float32:
+        return torch.mm(a, b)
+    ok = _MM_F32_OUT.get(a.device.type)
+    if ok is None and a.is_cuda:
+        try:
+            torch.mm(a[:1], b[:, :1], out_dtype=torch.float32)
+            ok = True
+        except (TypeError, RuntimeError):
+            ok = False
+        _MM_F32_OUT[a.device.type] = ok
+    return torch.mm(a, b, out_dtype=torch.float32) if ok else torch.mm(a.float(), b.float())
+
+
+# bytes of fp32 scores the product path holds at once
+PRODUCT_SCORE_BYTES = 256 << 20
+
+
+def latent_attention_products(out, qa, qr, cache, seg: Segments, scale: float, rank: int,
+                              min_rows: int, dtype):
+    """Segments of ``min_rows`` rows or more as two matrix products: all heads share
+    the cached rows, so with M = heads x rows the scores are Q [M, rank+dr] C^T and the
+    sums P [M, keys] C[:, :rank], with a causal softmax (fp32 statistics) in between.
+    Needs the segments' host copies; writes its rows of ``out`` [heads, T, rank]."""
+    start, pos0, kv_len = seg.host
+    heads = qa.shape[0]
+    bs = cache.shape[1]
+    width = cache.shape[2]
+    for s in range(seg.num):
+        a, b = start[s], start[s + 1]
+        n = b - a
+        if n < min_rows:
+            continue
+        nblk = (kv_len[s] + bs - 1) // bs
+        kv = cache.index_select(0, seg.block_tables[s, :nblk].long()).view(nblk * bs, width)
+        step = max(1, min(n, PRODUCT_SCORE_BYTES // (4 * heads * max(1, kv_len[s]))))
+        for c0 in range(0, n, step):
+            c1 = min(n, c0 + step)
+            keys = min(kv_len[s], pos0[s] + c1)          # the chunk's last row sees this many
+            q = torch.cat([qa[:, a + c0:a + c1], qr[a + c0:a + c1].transpose(0, 1)], -1) \
+                .reshape(heads * (c1 - c0), width).to(dtype)
+            sc = mm_f32(q, kv[:keys].t())
+            p = causal_softmax(sc, c1 - c0, pos0[s] + c0, scale, dtype)
+            out[:, a + c0:a + c1] = mm_f32(p, kv[:keys, :rank]).view(heads, c1 - c0, rank)
+    return out
 
 
 # ---------------------------------------------------------------------------------
@@ -205,6 +277,16 @@ def moe_topk(z, correction, top: int, groups: int, keep: int):
         native_mixers().moe_topk(idx, wts, z, correction, top, groups, keep)
         return idx, wts
     return ref.moe_topk(z, correction, top, groups, keep)
+
+
+def moe_pairs(out, h, idx, wts, wgu, wdown, limit: float):
+    """Few rows (decode): out (fp32, in place) += sum_k wts[:, k] * expert_{idx[:, k]}(h),
+    every (row, expert) pair streaming its expert's [gate | up] and down matrices; no
+    host round trip, so the step can be captured in a hipGraph."""
+    if out.is_cuda:
+        native_mixers().moe_pairs(out, h, idx, wts, wgu, wdown, float(limit))
+    else:
+        ref.moe_pairs(out, h, idx, wts, wgu, wdown, limit)
 
 
 def clamp_swiglu(gu, limit: float):

@@ -160,6 +160,14 @@ def latent_attention(qa, qr, cache, seg, scale, rank):
     return out
 
 
+def causal_softmax(s, rows_per_head, first_pos, scale, out_dtype):
+    rows, keys = s.shape
+    qpos = first_pos + torch.arange(rows, device=s.device) % rows_per_head
+    mask = torch.arange(keys, device=s.device)[None, :] <= qpos[:, None]
+    p = torch.softmax((s.float() * scale).masked_fill(~mask, float("-inf")), -1)
+    return p.masked_fill(~mask, 0.0).to(out_dtype)
+
+
 def moe_topk(z, correction, top, groups, keep):
     s = torch.softmax(z.float(), -1)
     ch = s + correction.float()
@@ -171,6 +179,14 @@ def moe_topk(z, correction, top, groups, keep):
         ch = ch.masked_fill(~gm.repeat_interleave(e // groups, 1), float("-inf"))
     idx = ch.topk(top, -1).indices
     return idx.int(), s.gather(1, idx)
+
+
+def moe_pairs(out, h, idx, wts, wgu, wdown, limit):
+    for t in range(h.shape[0]):
+        for k in range(idx.shape[1]):
+            e = int(idx[t, k])
+            y = clamp_swiglu(F.linear(h[t:t + 1], wgu[e]), limit)
+            out[t] += wts[t, k] * F.linear(y, wdown[e])[0].float()
 
 
 def clamp_swiglu(gu, limit, rows_scale=None):

@@ -77,11 +77,13 @@ def make_model(name, seed, tmp_path, tweak=None):
     return d, cfg, {k: v.float() for k, v in t.items()}
 
 
-def make_engine(ckpt, device, dtype="float32", pages=64, seqs=4, page=16):
+def make_engine(ckpt, device, dtype="float32", pages=64, seqs=4, page=16, graphs=False):
+    """``graphs``: decode steps replay captured graphs and are queued ahead (the
+    serving configuration on a GPU); otherwise every step runs eagerly."""
     return LLMEngine(EngineConfig(model=ckpt, weights=ckpt, device=device, dtype=dtype, num_kv_blocks=pages,
                                   block_size=page, max_num_seqs=seqs, max_model_len=pages * page,
-                                  max_num_batched_tokens=pages * page, enforce_eager=True,
-                                  async_output=False, swap_space_gb=0.0))
+                                  max_num_batched_tokens=pages * page, enforce_eager=not graphs,
+                                  async_output=graphs, swap_space_gb=0.0))
 
 
 def tokens(n, vocab, seed):

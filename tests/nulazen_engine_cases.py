@@ -101,11 +101,11 @@ def long_decode_persistent_state(device, dtype, tmp):
     assert (C.oracle(cfg, P, t2)[-1] - want[-1]).abs().max() > 1e-2
 
 
-def greedy_generation(name, device, dtype, tmp):
+def greedy_generation(name, device, dtype, tmp, graphs=False):
     """Through LLMEngine.generate: the scheduler's own batching, the sampler at
     temperature 0, against greedy decoding with the oracle."""
     d, cfg, P = C.make_model(name, 17, tmp)
-    eng = C.make_engine(d, device, dtype, seqs=2)     # three prompts, two slots: one waits
+    eng = C.make_engine(d, device, dtype, seqs=2, graphs=graphs)   # three prompts, two slots: one waits
     prompts = [C.tokens(n, cfg["vocab"], 50 + n) for n in (5, 1, 12)]
     outs = eng.generate(prompts, SamplingParams(temperature=0.0, max_tokens=7, ignore_eos=True))
     for p, out in zip(prompts, outs):
@@ -118,3 +118,5 @@ def greedy_generation(name, device, dtype, tmp):
                 assert lg[best] - lg[tok] < 1e-3, (seq, tok, best)
             seq.append(tok)
     assert eng.scheduler.slots.num_free() == 2
+    if graphs:
+        assert eng.runner.stats["graph_replays"] > 0

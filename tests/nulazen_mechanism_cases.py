@@ -8,7 +8,7 @@ import nulazen_oracle as O
 from fasttalk_llm_microservice_amd.models import mixers as X
 from fasttalk_llm_microservice_amd.ops import mixers as M
 
-CASES = ["rope", "norms", "latent", "latent_partial_rot", "delta", "delta_gqa_one_tap", "dense", "route",
+CASES = ["rope", "norms", "latent", "latent_partial_rot", "latent_products", "moe_pairs", "delta", "delta_gqa_one_tap", "dense", "route",
          "moe_shared", "moe_top1", "side"]
 EPS = 1e-5
 
@@ -17,7 +17,7 @@ def _rand(g, *shape, s=1.0):
     return (torch.randn(*shape, generator=g) * s).bfloat16().float()
 
 
-def _ctx(T, device, cut=None, page=4, slot=1):
+def _ctx(T, device, cut=None, page=4, slot=1, host=False):
     """StepContexts of one sequence of T rows: whole, or [0, cut) then [cut, T)."""
     i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=device)   # noqa: E731
     nb = (T + page - 1) // page
@@ -26,7 +26,8 @@ def _ctx(T, device, cut=None, page=4, slot=1):
     for a, b in ([(0, T)] if cut is None else [(0, cut), (cut, T)]):
         pos = list(range(a, b))
         seg = M.Segments(start=i32([0, b - a]), pos0=i32([a]), slot=i32([slot]), kv_len=i32([b]),
-                         block_tables=i32([table]), num=1, max_rows=b - a, max_kv=b)
+                         block_tables=i32([table]), num=1, max_rows=b - a, max_kv=b,
+                         host=([0, b - a], [a], [b]) if host else None)
         slots = [table[p // page] * page + p % page for p in pos]
         out.append((a, b, X.StepContext(None, i32(pos), i32(slots), seg)))
     return out
@@ -36,19 +37,20 @@ def _tol(dtype):
     return dict(rtol=3e-4, atol=3e-4) if dtype == torch.float32 else dict(rtol=6e-2, atol=6e-2)
 
 
-def _latent(device, dtype, dims):
+def _latent(device, dtype, dims, T=29, cuts=(None, 1, 13), host=False):
     g = torch.Generator().manual_seed(3)
-    W, T = 40, 29
+    W = 40
     m = {"heads": 3, "dim": 10, "rot_dim": 6, "vdim": 7, "kv_rank": 18, "scale": 0.35,
          "rot": {"base": 50.0, "dims": dims}}
     P = {"q": _rand(g, 3 * 16, W, s=0.4), "dkv": _rand(g, 24, W, s=0.3), "dkv.norm": 1 + _rand(g, 18, s=0.1),
          "uk": _rand(g, 30, 18, s=0.3), "uv": _rand(g, 21, 18, s=0.3), "o": _rand(g, W, 21, s=0.3)}
     h = _rand(g, T, W)
     want = O.latent_attention(h, P, "", m, EPS)
-    mix = X.LatentAttention(P.__getitem__, W, 3, 10, 6, 7, 18, 0.35, dims, 50.0, EPS, dtype, device, 64)
-    for cut in (None, 1, 13):
-        cache = torch.zeros(8, 4, 24, dtype=dtype, device=device)
-        got = torch.cat([mix(h[a:b].to(device, dtype), ctx, cache).float().cpu() for a, b, ctx in _ctx(T, device, cut)])
+    mix = X.LatentAttention(P.__getitem__, W, 3, 10, 6, 7, 18, 0.35, dims, 50.0, EPS, dtype, device, 128)
+    for cut in cuts:
+        cache = torch.zeros((T + 3) // 4, 4, 24, dtype=dtype, device=device)
+        got = torch.cat([mix(h[a:b].to(device, dtype), ctx, cache).float().cpu()
+                         for a, b, ctx in _ctx(T, device, cut, host=host)])
         torch.testing.assert_close(got, want, **_tol(dtype))
 
 
@@ -124,6 +126,30 @@ def run(case, device, dtype):
         _latent(device, dtype, 6)
     elif case == "latent_partial_rot":
         _latent(device, dtype, 2)
+    elif case == "latent_products":
+        # segments long enough for the matrix-product path, scores held in small pieces
+        old = M.PRODUCT_SCORE_BYTES
+        M.PRODUCT_SCORE_BYTES = 4 * 3 * 11 * 40
+        try:
+            _latent(device, dtype, 6, T=75, cuts=(None, 35, 3), host=True)
+        finally:
+            M.PRODUCT_SCORE_BYTES = old
+    elif case == "moe_pairs":
+        for (E, top, ff, W) in ((6, 2, 12, 32), (5, 3, 7, 19)):
+            wgu, wd = _rand(g, E, 2 * ff, W, s=0.5), _rand(g, E, W, ff, s=0.4)
+            h = _rand(g, 9, W)
+            idx = torch.stack([torch.randperm(E, generator=g)[:top] for _ in range(9)]).int()
+            wts = torch.rand(9, top, generator=g)
+            want = torch.zeros(9, W)
+            for t in range(9):
+                for k in range(top):
+                    e = int(idx[t, k])
+                    P = {"gate": wgu[e, :ff], "up": wgu[e, ff:], "down": wd[e]}
+                    want[t] += wts[t, k] * O.glu_expert(h[t:t + 1], P, "", 1.3)[0]
+            out = torch.zeros(9, W, device=device)
+            M.moe_pairs(out, h.to(device, dtype), idx.to(device), wts.to(device), wgu.to(device, dtype),
+                        wd.to(device, dtype), 1.3)
+            torch.testing.assert_close(out.cpu(), want, **_tol(dtype))
     elif case == "delta":
         _delta(device, dtype, 4, 2, 9, 11, 4)
     elif case == "delta_gqa_one_tap":

@@ -192,3 +192,13 @@ def test_moe_topk(experts, top, groups, keep):
     i2, w2 = M.moe_topk(z.to(DEV), corr.to(DEV), top, groups, keep)
     assert torch.equal(i2.cpu().sort(-1).values, i1.sort(-1).values)
     torch.testing.assert_close(w2.cpu().sort(-1).values, w1.sort(-1).values, rtol=1e-5, atol=1e-7)
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+def test_causal_softmax(dt):
+    g = torch.Generator().manual_seed(7)
+    s = rnd(3 * 5, 23, g=g, scale=3.0)
+    p1 = R.causal_softmax(s, 5, 17, 0.4, dt)
+    p2 = M.causal_softmax(s.to(DEV), 5, 17, 0.4, dt)
+    torch.testing.assert_close(p2.cpu().float(), p1.float(), **tol(dt))
+    assert float(p2[0, 18:].abs().max()) == 0.0 and float(p2[4, 22]) > 0.0

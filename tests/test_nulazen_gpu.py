@@ -51,6 +51,12 @@ def test_greedy_generation(name, tmp_path):
     E.greedy_generation(name, "cuda", "float32", tmp_path)
 
 
+@pytest.mark.parametrize("name", ["a", "b", "c"])
+def test_greedy_generation_graphs(name, tmp_path):
+    """Decode steps replayed from captured graphs and queued ahead of the host."""
+    E.greedy_generation(name, "cuda", "float32", tmp_path, graphs=True)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("case", K.CASES)
 def test_mechanism(case, dtype):
