@@ -3,6 +3,8 @@
 // As in csrc/bindings.cpp every op validates dtype / device / shape on the host (a
 // mis-shaped launch of a hand-written kernel can fault the GPU) and launches on the
 // caller's current stream without allocating or synchronising.
+#include <algorithm>
+
 #include <torch/extension.h>
 #include <c10/hip/HIPStream.h>
 #include <hip/hip_runtime.h>
@@ -44,6 +46,12 @@ int mx_latent_attention(float* out, const float* qa, const float* qr, const void
                         const int* start, const int* pos0, const int* kv_len, const int* bt, int bt_stride,
                         int num_segs, int max_rows, int heads, long total_rows, int rank, int dr,
                         int block_size, int num_blocks, float scale, int skip_from, hipStream_t s);
+long mx_latent_split_ws(int heads, int rank, int dr);
+int mx_latent_attention_split(float* out, float* ws_acc, float* ws_ml, const float* qa, const float* qr,
+                              const void* cache, int cache_bf16, const int* start, const int* pos0,
+                              const int* kv_len, const int* bt, int bt_stride, int num_segs, int max_rows,
+                              int heads, long total_rows, int rank, int dr, int block_size, int num_blocks,
+                              float scale, int skip_from, int splits, hipStream_t s);
 int mx_causal_softmax(void* P, int p_bf16, const float* S, long rows, int rows_per_head, int first_pos, int ncols,
                       float scale, hipStream_t s);
 int mx_moe_pairs(float* out, void* y, const void* h, int bf16, long h_stride, const int* idx, const float* wts,
@@ -267,7 +275,8 @@ void latent_q_rope(Tensor qn, Tensor qr, Tensor q, Tensor table, int64_t dims, T
 }
 
 void latent_attention(Tensor out, Tensor qa, Tensor qr, Tensor cache, Tensor start, Tensor pos0, Tensor kv_len,
-                      Tensor bt, int64_t num_segs, int64_t max_rows, double scale, int64_t rank, int64_t skip_from) {
+                      Tensor bt, int64_t num_segs, int64_t max_rows, double scale, int64_t rank, int64_t skip_from,
+                      int64_t max_kv) {
   check_f32(out, "out");
   check_f32(qa, "qa");
   check_f32(qr, "qr");
@@ -279,6 +288,23 @@ void latent_attention(Tensor out, Tensor qa, Tensor qr, Tensor cache, Tensor sta
   check_segs(start, pos0, kv_len, num_segs);
   check_i32(bt, "block tables");
   TORCH_CHECK(bt.dim() == 2 && bt.size(0) >= num_segs && max_rows <= t, "block tables / max_rows");
+  if (mx_latent_split_ws((int)heads, (int)rank, (int)dr)) {
+    // key slices: enough workgroups to fill the chip, at least ~64 keys per slice when
+    // the longest context is known (max_kv; 0 inside captured graphs), scratch <= 256 MiB
+    int64_t rows = std::max<int64_t>(1, std::min<int64_t>(t, num_segs * std::max<int64_t>(1, std::min(max_rows, skip_from > 0 ? skip_from - 1 : max_rows))));
+    int64_t splits = std::max<int64_t>(1, std::min<int64_t>(32, 512 / rows));
+    if (max_kv > 0) splits = std::max<int64_t>(1, std::min(splits, (max_kv + 63) / 64));
+    while (splits > 1 && t * splits * heads * rank * 4 > (256LL << 20)) splits /= 2;
+    auto f32 = qa.options();
+    Tensor ws_acc = at::empty({t, splits, heads, rank}, f32), ws_ml = at::empty({t, splits, heads, 2}, f32);
+    chk(mx_latent_attention_split(out.data_ptr<float>(), ws_acc.data_ptr<float>(), ws_ml.data_ptr<float>(),
+                                  qa.data_ptr<float>(), qr.data_ptr<float>(), cache.data_ptr(), bf(cache),
+                                  start.data_ptr<int>(), pos0.data_ptr<int>(), kv_len.data_ptr<int>(),
+                                  bt.data_ptr<int>(), (int)bt.size(1), (int)num_segs, (int)max_rows, (int)heads,
+                                  t, (int)rank, (int)dr, (int)cache.size(1), (int)cache.size(0), (float)scale,
+                                  (int)skip_from, (int)splits, stream()), "latent_attention_split");
+    return;
+  }
   chk(mx_latent_attention(out.data_ptr<float>(), qa.data_ptr<float>(), qr.data_ptr<float>(), cache.data_ptr(),
                           bf(cache), start.data_ptr<int>(), pos0.data_ptr<int>(), kv_len.data_ptr<int>(),
                           bt.data_ptr<int>(), (int)bt.size(1), (int)num_segs, (int)max_rows, (int)heads, t,

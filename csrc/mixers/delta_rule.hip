@@ -9,9 +9,9 @@
 // Recurrence per head, S [dk, dv] fp32:
 //   S <- diag(g) S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
 // Columns of S (the dv axis) are independent, so a workgroup owns 32 columns of one
-// head of one sequence: 8 lanes share a column (each holds dk/8 rows in registers, the
-// two dot products are reduced over those 8 lanes), and the rows of a segment are
-// walked in order.  q, k (unit-normalised), g and beta are prepared for all rows at
+// head of one sequence: 8 lanes share a column (each holds dk/8 consecutive rows in
+// registers, the two dot products are reduced over those 8 lanes), and the rows of a
+// segment are walked in order.  q, k (unit-normalised), g and beta are prepared for all rows at
 // once by delta_prep_kernel, so the sequential loop only streams them.
 #include "mx_common.h"
 
@@ -121,7 +121,39 @@ __global__ void delta_prep_kernel(float* __restrict__ qn, float* __restrict__ kn
 constexpr int kKL = 8;        // lanes that share one state column
 constexpr int kCols = 32;     // state columns per workgroup (256 threads)
 
-// grid (dv tiles, heads, segments), 256 threads; R = state rows per thread (dk <= 8 R)
+// sum over the 8 adjacent lanes that share a column, on the VALU's lane-permute path
+// (quad swaps, then the mirrored half row): every lane of the group gets the total
+__device__ __forceinline__ float sum8(float v) {
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, true));   // lanes ^ 1
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xF, 0xF, true));   // lanes ^ 2
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xF, 0xF, true));  // 7 - lane
+  return v;
+}
+
+// a thread's R consecutive entries of a per-row vector (zeros past dk)
+template <int R>
+__device__ __forceinline__ void load_rows(float (&dst)[R], const float* __restrict__ src, int i0, int dk,
+                                          bool vec) {
+  if (vec) {
+#pragma unroll
+    for (int r = 0; r < R; r += 4) {
+      if (i0 + r < dk) {
+        const float4 v = *reinterpret_cast<const float4*>(src + i0 + r);
+        dst[r] = v.x; dst[r + 1] = v.y; dst[r + 2] = v.z; dst[r + 3] = v.w;
+      } else {
+        dst[r] = dst[r + 1] = dst[r + 2] = dst[r + 3] = 0.f;
+      }
+    }
+  } else {
+#pragma unroll
+    for (int r = 0; r < R; ++r) dst[r] = i0 + r < dk ? src[i0 + r] : 0.f;
+  }
+}
+
+// grid (dv tiles, heads, segments), 256 threads.  Lane group member kl holds the state
+// rows [kl R, kl R + R) of its column (dk <= 8 R).  The next row's q, k, decay, v and
+// beta are fetched while the current row is computed, so the loop-carried chain is the
+// state update alone.
 template <typename T, int R>
 __global__ void __launch_bounds__(256)
 delta_rule_kernel(float* __restrict__ o, const float* __restrict__ qn, const float* __restrict__ kn,
@@ -144,48 +176,63 @@ delta_rule_kernel(float* __restrict__ o, const float* __restrict__ qn, const flo
   }
   if (n <= 0) return;
   const int kh = h / (heads / kv_heads);
+  const int i0 = kl * R;
+  const bool vec = (R % 4 == 0) && (dk % 4 == 0);
   float* S = state + (((long)sl * heads + h) * dk) * dv;
   float st_[R];
   const bool fresh = pos0[s] <= 0;
 #pragma unroll
-  for (int r = 0; r < R; ++r) {
-    const int i = kl + kKL * r;
-    st_[r] = (!fresh && i < dk) ? S[(long)i * dv + c] : 0.f;
-  }
+  for (int r = 0; r < R; ++r) st_[r] = (!fresh && i0 + r < dk) ? S[(long)(i0 + r) * dv + c] : 0.f;
   const long voff = 2L * kv_heads * dk + (long)h * dv + c;
+  float kk[R], qq[R], gg[R], nk[R], nq[R], ng[R];
+  float vv, bb, nv = 0.f, nb = 0.f;
+  {
+    const long row = r0;
+    load_rows<R>(nk, kn + (row * kv_heads + kh) * dk, i0, dk, vec);
+    load_rows<R>(nq, qn + (row * kv_heads + kh) * dk, i0, dk, vec);
+    load_rows<R>(ng, g + (row * heads + h) * dk, i0, dk, vec);
+    nv = ld(qkv, row * qkv_stride + voff);
+    nb = beta[row * heads + h];
+  }
   for (int t = 0; t < n; ++t) {
     const long row = r0 + t;
-    const float* qp = qn + (row * kv_heads + kh) * dk;
-    const float* kp = kn + (row * kv_heads + kh) * dk;
-    const float* gp = g + (row * heads + h) * dk;
-    float kk[R], qq[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      kk[r] = nk[r];
+      qq[r] = nq[r];
+      gg[r] = ng[r];
+    }
+    vv = nv;
+    bb = nb;
+    if (t + 1 < n) {
+      const long nx = row + 1;
+      load_rows<R>(nk, kn + (nx * kv_heads + kh) * dk, i0, dk, vec);
+      load_rows<R>(nq, qn + (nx * kv_heads + kh) * dk, i0, dk, vec);
+      load_rows<R>(ng, g + (nx * heads + h) * dk, i0, dk, vec);
+      nv = ld(qkv, nx * qkv_stride + voff);
+      nb = beta[nx * heads + h];
+    }
     float dot = 0.f;
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-      const int i = kl + kKL * r;
-      const bool in = i < dk;
-      kk[r] = in ? kp[i] : 0.f;
-      qq[r] = in ? qp[i] : 0.f;
-      st_[r] *= in ? gp[i] : 0.f;
+      st_[r] *= gg[r];
       dot += st_[r] * kk[r];
     }
-    dot = ft::group_sum<kKL>(dot);
-    const float u = beta[row * heads + h] * (ld(qkv, row * qkv_stride + voff) - dot);
+    dot = sum8(dot);
+    const float u = bb * (vv - dot);
     float out = 0.f;
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       st_[r] += kk[r] * u;
       out += st_[r] * qq[r];
     }
-    out = ft::group_sum<kKL>(out);
+    out = sum8(out);
     if (live && kl == 0) o[row * o_stride + (long)h * dv + col] = out;
   }
   if (live) {
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-      const int i = kl + kKL * r;
-      if (i < dk) S[(long)i * dv + col] = st_[r];
-    }
+    for (int r = 0; r < R; ++r)
+      if (i0 + r < dk) S[(long)(i0 + r) * dv + col] = st_[r];
   }
 }
 

@@ -147,6 +147,143 @@ latent_attention_kernel(float* __restrict__ out, const float* __restrict__ qa, c
   }
 }
 
+// ---------------------------------------------------------------------------------
+// Split-key kernel for decode rows and short segments.  A workgroup owns (one query
+// row, one slice of its keys, one group of up to 16 heads): it stages tiles of cache
+// rows in LDS (coalesced, widened to fp32, odd row stride against bank conflicts) and
+// every head of the group scores and accumulates against the same tile, so a cache row
+// is read once per head group instead of once per head.  Each workgroup leaves (max,
+// sum, weighted c sums) per head; latent_combine_kernel merges the slices.
+// ---------------------------------------------------------------------------------
+template <typename TC, int ACC>
+__global__ void __launch_bounds__(256)
+latent_split_kernel(float* __restrict__ ws_acc, float* __restrict__ ws_ml, const float* __restrict__ qa,
+                    const float* __restrict__ qr, const TC* __restrict__ cache, const int* __restrict__ start,
+                    const int* __restrict__ pos0, const int* __restrict__ kv_len, const int* __restrict__ bt,
+                    int bt_stride, int heads, long total_rows, int rank, int dr, int block_size,
+                    int num_blocks, float scale, int skip_from, int splits, int hg, int tk) {
+  extern __shared__ float smem[];
+  const int s = blockIdx.z;
+  const int r0 = start[s], n = start[s + 1] - r0;
+  const int rel = blockIdx.y;
+  if (rel >= n || (skip_from > 0 && n >= skip_from)) return;
+  const long row = r0 + rel;
+  const int sp = blockIdx.x % splits, h0 = (blockIdx.x / splits) * hg;
+  const int nh = min(hg, heads - h0);
+  const int width = rank + dr, ldk = width | 1;
+  float* qs = smem;                       // [hg, width]
+  float* kt = qs + hg * width;            // [tk, ldk]
+  float* ps = kt + tk * ldk;              // [hg, tk]
+  float* ms = ps + hg * tk;               // [hg] running max
+  float* ls = ms + hg;                    // [hg] running sum
+  float* al = ls + hg;                    // [hg] rescale of this tile
+  const int tid = threadIdx.x;
+  int nk = pos0[s] + rel + 1;
+  if (nk > kv_len[s]) nk = kv_len[s];
+  const int per = (nk + splits - 1) / splits;
+  const int chunk = (per + tk - 1) / tk * tk;
+  const int k_begin = sp * chunk, k_end = min(nk, k_begin + chunk);
+  const int* tab = bt + (long)s * bt_stride;
+  for (int e = tid; e < nh * width; e += 256) {
+    const int h = e / width, i = e % width;
+    qs[e] = i < rank ? qa[((long)(h0 + h) * total_rows + row) * rank + i]
+                     : qr[(row * heads + h0 + h) * dr + (i - rank)];
+  }
+  if (tid < hg) {
+    ms[tid] = -INFINITY;
+    ls[tid] = 0.f;
+  }
+  float acc[ACC];
+#pragma unroll
+  for (int a = 0; a < ACC; ++a) acc[a] = 0.f;
+  for (int k0 = k_begin; k0 < k_end; k0 += tk) {
+    const int cnt = min(tk, k_end - k0);
+    __syncthreads();                      // the previous tile is no longer read
+    for (int e = tid; e < cnt * width; e += 256) {
+      const int j = e / width, i = e % width;
+      const int tok = k0 + j;
+      int blk = tab[tok / block_size];
+      if (blk < 0 || blk >= num_blocks) blk = 0;
+      kt[j * ldk + i] = ld(cache, ((long)blk * block_size + tok % block_size) * width + i);
+    }
+    __syncthreads();
+    for (int p = tid; p < nh * cnt; p += 256) {
+      const int h = p / cnt, j = p % cnt;
+      const float* q = qs + h * width;
+      const float* k = kt + j * ldk;
+      float d = 0.f;
+      for (int i = 0; i < width; ++i) d += q[i] * k[i];
+      ps[h * tk + j] = d * scale;
+    }
+    __syncthreads();
+    if (tid < nh) {
+      float* pr = ps + tid * tk;
+      float mt = -INFINITY;
+      for (int j = 0; j < cnt; ++j) mt = fmaxf(mt, pr[j]);
+      const float mo = ms[tid], mn = fmaxf(mo, mt);
+      float sum = 0.f;
+      for (int j = 0; j < cnt; ++j) {
+        const float e = expf(pr[j] - mn);
+        pr[j] = e;
+        sum += e;
+      }
+      const float a = expf(mo - mn);      // 0 at the first tile (mo = -inf)
+      al[tid] = a;
+      ls[tid] = ls[tid] * a + sum;
+      ms[tid] = mn;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int a = 0; a < ACC; ++a) {
+      const int o = tid + 256 * a;
+      if (o < nh * rank) {
+        const int h = o / rank, d = o % rank;
+        float v = acc[a] * al[h];
+        const float* pr = ps + h * tk;
+        for (int j = 0; j < cnt; ++j) v += pr[j] * kt[j * ldk + d];
+        acc[a] = v;
+      }
+    }
+  }
+  __syncthreads();
+  const long base = (row * splits + sp) * heads + h0;
+#pragma unroll
+  for (int a = 0; a < ACC; ++a) {
+    const int o = tid + 256 * a;
+    if (o < nh * rank) ws_acc[(base + o / rank) * rank + o % rank] = acc[a];
+  }
+  if (tid < nh) {
+    ws_ml[(base + tid) * 2] = ms[tid];
+    ws_ml[(base + tid) * 2 + 1] = ls[tid];
+  }
+}
+
+// out[h, row, :] = sum_s exp(m_s - M) acc_s / sum_s exp(m_s - M) l_s over the key slices
+__global__ void latent_combine_kernel(float* __restrict__ out, const float* __restrict__ ws_acc,
+                                      const float* __restrict__ ws_ml, const int* __restrict__ start,
+                                      int heads, long total_rows, int rank, int skip_from, int splits) {
+  const int s = blockIdx.y;
+  const int r0 = start[s], n = start[s + 1] - r0;
+  const int rel = blockIdx.x;
+  if (rel >= n || (skip_from > 0 && n >= skip_from)) return;
+  const long row = r0 + rel;
+  for (int o = threadIdx.x; o < heads * rank; o += blockDim.x) {
+    const int h = o / rank, d = o % rank;
+    float M = -INFINITY;
+    for (int sp = 0; sp < splits; ++sp) M = fmaxf(M, ws_ml[((row * splits + sp) * heads + h) * 2]);
+    float L = 0.f, v = 0.f;
+    for (int sp = 0; sp < splits; ++sp) {
+      const long b = (row * splits + sp) * heads + h;
+      const float m = ws_ml[b * 2];
+      if (m == -INFINITY) continue;       // an empty slice
+      const float w = expf(m - M);
+      L += w * ws_ml[b * 2 + 1];
+      v += w * ws_acc[b * rank + d];
+    }
+    out[((long)h * total_rows + row) * rank + d] = L > 0.f ? v / L : 0.f;
+  }
+}
+
 // P[r, j] = softmax_j(scale * S[r, j]) over the keys j <= first_pos + (r mod rows_per_head),
 // 0 beyond (rows r = head * rows_per_head + query row); fp32 statistics, P in TP
 template <typename TP, int NT>
@@ -262,5 +399,79 @@ extern "C" int mx_latent_attention(float* out, const float* qa, const float* qr,
   else if (need <= 8) MX_LAT(8);
   else MX_LAT(16);
 #undef MX_LAT
+  return (int)hipGetLastError();
+}
+
+// plan of the split-key kernel for these sizes: heads per group, keys per tile, LDS
+// bytes, accumulators per thread (0: does not fit, use the per-row kernel)
+static int split_plan(int heads, int rank, int dr, int* hg, int* tk, size_t* lds) {
+  const int width = rank + dr, ldk = width | 1;
+  int g = heads < 16 ? heads : 16;
+  while (g > 1 && (long)g * width > 9216) --g;
+  const long budget = 64 * 1024 / 4 - 64;
+  long t = (budget - (long)g * width - 3 * g) / (ldk + g);
+  if (t < 2) return 0;
+  if (t > 32) t = 32;
+  const int acc = (g * rank + 255) / 256;
+  if (acc > 64) return 0;
+  *hg = g;
+  *tk = (int)t;
+  *lds = (size_t)(g * width + t * ldk + g * t + 3 * g) * sizeof(float);
+  return acc;
+}
+
+extern "C" long mx_latent_split_ws(int heads, int rank, int dr) {
+  int hg, tk;
+  size_t lds;
+  return split_plan(heads, rank, dr, &hg, &tk, &lds) ? 1 : 0;
+}
+
+template <typename TC, int ACC>
+static void launch_split(dim3 grid, size_t lds, hipStream_t s, float* ws_acc, float* ws_ml, const float* qa,
+                         const float* qr, const void* cache, const int* start, const int* pos0,
+                         const int* kv_len, const int* bt, int bt_stride, int heads, long total_rows, int rank,
+                         int dr, int block_size, int num_blocks, float scale, int skip_from, int splits, int hg,
+                         int tk) {
+  hipLaunchKernelGGL((latent_split_kernel<TC, ACC>), grid, dim3(256), lds, s, ws_acc, ws_ml, qa, qr,
+                     (const TC*)cache, start, pos0, kv_len, bt, bt_stride, heads, total_rows, rank, dr,
+                     block_size, num_blocks, scale, skip_from, splits, hg, tk);
+}
+
+extern "C" int mx_latent_attention_split(float* out, float* ws_acc, float* ws_ml, const float* qa,
+                                         const float* qr, const void* cache, int cache_bf16, const int* start,
+                                         const int* pos0, const int* kv_len, const int* bt, int bt_stride,
+                                         int num_segs, int max_rows, int heads, long total_rows, int rank,
+                                         int dr, int block_size, int num_blocks, float scale, int skip_from,
+                                         int splits, hipStream_t s) {
+  if (num_segs <= 0 || max_rows <= 0) return 0;
+  if (skip_from > 0 && max_rows >= skip_from) max_rows = skip_from - 1;
+  if (max_rows <= 0) return 0;
+  int hg, tk;
+  size_t lds;
+  const int acc = split_plan(heads, rank, dr, &hg, &tk, &lds);
+  if (!acc || splits < 1 || max_rows > 65535 || num_segs > 65535) return -1;
+  const int groups = (heads + hg - 1) / hg;
+  const dim3 grid(splits * groups, max_rows, num_segs);
+#define MX_SPLIT(A)                                                                                      \
+  do {                                                                                                   \
+    if (cache_bf16)                                                                                      \
+      launch_split<bf16_t, A>(grid, lds, s, ws_acc, ws_ml, qa, qr, cache, start, pos0, kv_len, bt,       \
+                              bt_stride, heads, total_rows, rank, dr, block_size, num_blocks, scale,     \
+                              skip_from, splits, hg, tk);                                                \
+    else                                                                                                 \
+      launch_split<float, A>(grid, lds, s, ws_acc, ws_ml, qa, qr, cache, start, pos0, kv_len, bt,        \
+                             bt_stride, heads, total_rows, rank, dr, block_size, num_blocks, scale,      \
+                             skip_from, splits, hg, tk);                                                 \
+  } while (0)
+  if (acc <= 1) MX_SPLIT(1);
+  else if (acc <= 2) MX_SPLIT(2);
+  else if (acc <= 4) MX_SPLIT(4);
+  else if (acc <= 8) MX_SPLIT(8);
+  else if (acc <= 16) MX_SPLIT(16);
+  else if (acc <= 32) MX_SPLIT(32);
+  else MX_SPLIT(64);
+#undef MX_SPLIT
+  hipLaunchKernelGGL(latent_combine_kernel, dim3(max_rows, num_segs), dim3(256), 0, s, out, ws_acc, ws_ml,
+                     start, heads, total_rows, rank, skip_from, splits);
   return (int)hipGetLastError();
 }

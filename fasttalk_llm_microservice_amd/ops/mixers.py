@@ -191,7 +191,7 @@ def latent_attention(qa, qr, cache, seg: Segments, scale: float, rank: int,
             out = torch.empty_like(qa)
         native_mixers().latent_attention(out, qa, qr, cache, seg.start, seg.pos0, seg.kv_len,
                                          seg.block_tables, seg.num, seg.max_rows, scale, rank,
-                                         skip_from)
+                                         skip_from, seg.max_kv)
         return out
     r = ref.latent_attention(qa, qr, cache, seg, scale, rank)
     if out is not None:
