@@ -170,9 +170,9 @@ latent_split_kernel(float* __restrict__ ws_acc, float* __restrict__ ws_ml, const
   const long row = r0 + rel;
   const int sp = blockIdx.x % splits, h0 = (blockIdx.x / splits) * hg;
   const int nh = min(hg, heads - h0);
-  const int width = rank + dr, ldk = width | 1;
-  float* qs = smem;                       // [hg, width]
-  float* kt = qs + hg * width;            // [tk, ldk]
+  const int width = rank + dr, ldk = width | 1;   // odd strides: heads / keys land on different banks
+  float* qs = smem;                       // [hg, ldk]
+  float* kt = qs + hg * ldk;              // [tk, ldk]
   float* ps = kt + tk * ldk;              // [hg, tk]
   float* ms = ps + hg * tk;               // [hg] running max
   float* ls = ms + hg;                    // [hg] running sum
@@ -186,7 +186,7 @@ latent_split_kernel(float* __restrict__ ws_acc, float* __restrict__ ws_ml, const
   const int* tab = bt + (long)s * bt_stride;
   for (int e = tid; e < nh * width; e += 256) {
     const int h = e / width, i = e % width;
-    qs[e] = i < rank ? qa[((long)(h0 + h) * total_rows + row) * rank + i]
+    qs[h * ldk + i] = i < rank ? qa[((long)(h0 + h) * total_rows + row) * rank + i]
                      : qr[(row * heads + h0 + h) * dr + (i - rank)];
   }
   if (tid < hg) {
@@ -209,7 +209,7 @@ latent_split_kernel(float* __restrict__ ws_acc, float* __restrict__ ws_ml, const
     __syncthreads();
     for (int p = tid; p < nh * cnt; p += 256) {
       const int h = p / cnt, j = p % cnt;
-      const float* q = qs + h * width;
+      const float* q = qs + h * ldk;
       const float* k = kt + j * ldk;
       float d = 0.f;
       for (int i = 0; i < width; ++i) d += q[i] * k[i];
@@ -267,8 +267,8 @@ __global__ void latent_combine_kernel(float* __restrict__ out, const float* __re
   const int rel = blockIdx.x;
   if (rel >= n || (skip_from > 0 && n >= skip_from)) return;
   const long row = r0 + rel;
-  for (int o = threadIdx.x; o < heads * rank; o += blockDim.x) {
-    const int h = o / rank, d = o % rank;
+  const int h = blockIdx.z;
+  for (int d = threadIdx.x; d < rank; d += blockDim.x) {
     float M = -INFINITY;
     for (int sp = 0; sp < splits; ++sp) M = fmaxf(M, ws_ml[((row * splits + sp) * heads + h) * 2]);
     float L = 0.f, v = 0.f;
@@ -407,16 +407,16 @@ extern "C" int mx_latent_attention(float* out, const float* qa, const float* qr,
 static int split_plan(int heads, int rank, int dr, int* hg, int* tk, size_t* lds) {
   const int width = rank + dr, ldk = width | 1;
   int g = heads < 16 ? heads : 16;
-  while (g > 1 && (long)g * width > 9216) --g;
+  while (g > 1 && (long)g * ldk > 9300) --g;
   const long budget = 64 * 1024 / 4 - 64;
-  long t = (budget - (long)g * width - 3 * g) / (ldk + g);
+  long t = (budget - (long)g * ldk - 3 * g) / (ldk + g);
   if (t < 2) return 0;
   if (t > 32) t = 32;
   const int acc = (g * rank + 255) / 256;
   if (acc > 64) return 0;
   *hg = g;
   *tk = (int)t;
-  *lds = (size_t)(g * width + t * ldk + g * t + 3 * g) * sizeof(float);
+  *lds = (size_t)(g * ldk + t * ldk + g * t + 3 * g) * sizeof(float);
   return acc;
 }
 
@@ -449,7 +449,7 @@ extern "C" int mx_latent_attention_split(float* out, float* ws_acc, float* ws_ml
   int hg, tk;
   size_t lds;
   const int acc = split_plan(heads, rank, dr, &hg, &tk, &lds);
-  if (!acc || splits < 1 || max_rows > 65535 || num_segs > 65535) return -1;
+  if (!acc || splits < 1 || max_rows > 65535 || num_segs > 65535 || heads > 65535) return -1;
   const int groups = (heads + hg - 1) / hg;
   const dim3 grid(splits * groups, max_rows, num_segs);
 #define MX_SPLIT(A)                                                                                      \
@@ -471,7 +471,7 @@ extern "C" int mx_latent_attention_split(float* out, float* ws_acc, float* ws_ml
   else if (acc <= 32) MX_SPLIT(32);
   else MX_SPLIT(64);
 #undef MX_SPLIT
-  hipLaunchKernelGGL(latent_combine_kernel, dim3(max_rows, num_segs), dim3(256), 0, s, out, ws_acc, ws_ml,
-                     start, heads, total_rows, rank, skip_from, splits);
+  hipLaunchKernelGGL(latent_combine_kernel, dim3(max_rows, num_segs, heads), dim3(rank >= 256 ? 256 : 64), 0,
+                     s, out, ws_acc, ws_ml, start, heads, total_rows, rank, skip_from, splits);
   return (int)hipGetLastError();
 }

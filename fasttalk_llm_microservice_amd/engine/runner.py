@@ -683,7 +683,7 @@ class ModelRunner:
             if not has_logits:
                 self._wait() if self.is_gpu else None
                 return np.zeros((0, self.mcfg.vocab_size), np.float32)
-            logits = self.model.compute_logits(h).float()
+            logits = self.model.compute_logits(h).float()[:, :self.mcfg.vocab_size]
             if not self.is_gpu:
                 return logits.numpy()
             out = torch.empty(logits.shape, dtype=torch.float32, pin_memory=True)

@@ -257,7 +257,13 @@ class NulazenModel:
         eps = cfg.rms_norm_eps
         f32 = lambda n: get(n).to(dev, torch.float32)   # noqa: E731
         self.embed = get("embed").to(dev, dt).contiguous()
-        self.head = get("head").to(dev, dt).contiguous()
+        head = get("head").to(dev, dt)
+        # the sampler reads logits rows in groups of 8: zero rows pad the head, and their
+        # logits are set to -inf (never sampled; callers that want logits cut them off)
+        self.vocab_pad = (-head.shape[0]) % 8
+        if self.vocab_pad:
+            head = torch.cat([head, torch.zeros(self.vocab_pad, head.shape[1], dtype=dt, device=dev)], 0)
+        self.head = head.contiguous()
         self.final_norm = f32("final.norm")
         self.loop_step = f32("loop.step") if cfg.loop else None
         self.side_embed = get("side.embed").to(dev, dt).contiguous() if cfg.side_dim else None
@@ -392,7 +398,14 @@ class NulazenModel:
         return M.rms_norm_rows(rows, self.final_norm, eps, dt)
 
     def compute_logits(self, h: torch.Tensor) -> torch.Tensor:
-        """fp32 logits [rows, vocab]."""
+        """fp32 logits [rows, vocab rounded up to a multiple of 8]; columns past the
+        vocabulary are -inf."""
+        logits = self._head_product(h)
+        if self.vocab_pad:
+            logits[:, self.cfg.vocab_size:] = float("-inf")
+        return logits
+
+    def _head_product(self, h: torch.Tensor) -> torch.Tensor:
         if h.dtype == torch.float32:
             return F.linear(h, self.head)
         # bf16 operands, fp32 accumulation and fp32 output

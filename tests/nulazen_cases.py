@@ -62,6 +62,15 @@ CONFIGS = {
                "mlp": _moe(8, 3, 12, 1.0, groups=(2, 1), shared=(16, 2.0))},
               {"type": "channel_delta", "mixer": _delta(5, 5, 4, 6, 5), "mlp": _moe(4, 4, 8, 3.0)}],
           "loop": {"start": 1, "stop": 3, "times": 3}, "token_side": {"dim": 3}},
+    # dense feed-forwards only: bf16 runs are compared with the fp32 oracle on this one (a
+    # routing choice that flips under bf16 rounding changes a row's output entirely, so
+    # bf16 expert layers are checked per mechanism instead)
+    "d": {"architecture": "Nulazen", "vocab": 90, "width": 64, "norm": {"eps": 1e-5},
+          "layers": [
+              {"type": "channel_delta", "mixer": _delta(4, 2, 16, 8, 3), "mlp": {"kind": "dense", "ff": 80}},
+              {"type": "latent_attention", "mixer": _latent(2, 16, 8, 8, 12, 24, 0.2), "mlp": {"kind": "dense", "ff": 72}},
+              {"type": "channel_delta", "mixer": _delta(2, 2, 8, 16, 2), "mlp": None}],
+          "loop": {"start": 1, "stop": 3, "times": 2}, "token_side": {"dim": 4}},
 }
 
 
@@ -118,7 +127,7 @@ def close(got, want, dtype="float32"):
         return
     # bf16: rounding differs from the fp32 oracle everywhere, and a routing choice can flip
     err = (got - want).pow(2).mean(-1).sqrt() / want.pow(2).mean(-1).sqrt().clamp_min(1e-3)
-    assert err.median() < 0.08 and (err > 0.3).float().mean() <= 0.1, err
+    assert err.median() < 0.1 and err.max() < 0.4, err
 
 
 def oracle(cfg, P, toks):
