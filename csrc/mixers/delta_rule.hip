@@ -11,8 +11,8 @@
 // Columns of S (the dv axis) are independent, so a workgroup owns 32 columns of one
 // head of one sequence: 8 lanes share a column (each holds dk/8 consecutive rows in
 // registers, the two dot products are reduced over those 8 lanes), and the rows of a
-// segment are walked in order.  q, k (unit-normalised), g and beta are prepared for all rows at
-// once by delta_prep_kernel, so the sequential loop only streams them.
+// segment are walked in order.  q, k (unit-normalised), g and beta are prepared for all
+// rows at once by delta_prep_kernel, so the sequential loop only streams them.
 #include "mx_common.h"
 
 namespace mx {
@@ -130,30 +130,23 @@ __device__ __forceinline__ float sum8(float v) {
   return v;
 }
 
-// a thread's R consecutive entries of a per-row vector (zeros past dk)
-template <int R>
-__device__ __forceinline__ void load_rows(float (&dst)[R], const float* __restrict__ src, int i0, int dk,
-                                          bool vec) {
-  if (vec) {
-#pragma unroll
-    for (int r = 0; r < R; r += 4) {
-      if (i0 + r < dk) {
-        const float4 v = *reinterpret_cast<const float4*>(src + i0 + r);
-        dst[r] = v.x; dst[r + 1] = v.y; dst[r + 2] = v.z; dst[r + 3] = v.w;
-      } else {
-        dst[r] = dst[r + 1] = dst[r + 2] = dst[r + 3] = 0.f;
-      }
-    }
-  } else {
-#pragma unroll
-    for (int r = 0; r < R; ++r) dst[r] = i0 + r < dk ? src[i0 + r] : 0.f;
-  }
-}
-
 // grid (dv tiles, heads, segments), 256 threads.  Lane group member kl holds the state
-// rows [kl R, kl R + R) of its column (dk <= 8 R).  The next row's q, k, decay, v and
-// beta are fetched while the current row is computed, so the loop-carried chain is the
-// state update alone.
+// rows kl, kl + 8, ... of its column (dk <= 8 R).
+//
+// The per-row inputs (k, q, decay: dk floats each; v: this tile's 32 columns; beta) are
+// staged through LDS in chunks of TT rows, double buffered: all 256 threads issue the
+// next chunk's global loads before the current chunk's rows are walked and park them in
+// LDS afterwards, so the sequential loop reads LDS only and one memory latency is paid
+// per TT rows, overlapped with the walk.
+template <int R>
+struct DeltaTile {
+  static constexpr int TT = R <= 16 ? 16 : 8;                 // rows per chunk
+  static constexpr int DKP = 8 * R;                           // padded key size
+  static constexpr int ROWF = 3 * DKP + kCols + 1;            // floats per staged row
+  static constexpr int NLD = (TT * 3 * DKP + 255) / 256;      // k/q/g loads per thread and chunk
+  static constexpr int NV = (TT * kCols + 255) / 256;         // v loads per thread and chunk
+};
+
 template <typename T, int R>
 __global__ void __launch_bounds__(256)
 delta_rule_kernel(float* __restrict__ o, const float* __restrict__ qn, const float* __restrict__ kn,
@@ -161,11 +154,15 @@ delta_rule_kernel(float* __restrict__ o, const float* __restrict__ qn, const flo
                   long qkv_stride, float* __restrict__ state, const int* __restrict__ start,
                   const int* __restrict__ pos0, const int* __restrict__ slot, int heads, int kv_heads,
                   int dk, int dv, int num_slots) {
+  using P = DeltaTile<R>;
+  __shared__ float stage[2][P::TT * P::ROWF];
   const int s = blockIdx.z, h = blockIdx.y;
   const int sl = slot[s];
   const int r0 = start[s], n = start[s + 1] - r0;
-  const int kl = threadIdx.x & (kKL - 1);
-  const int col = blockIdx.x * kCols + (threadIdx.x >> 3);
+  const int tid = threadIdx.x;
+  const int kl = tid & (kKL - 1);
+  const int cl = tid >> 3;                // column within the tile
+  const int col = blockIdx.x * kCols + cl;
   const bool live = col < dv;
   const int c = live ? col : dv - 1;      // dead lanes shadow the last column, store nothing
   const long o_stride = (long)heads * dv;
@@ -176,63 +173,94 @@ delta_rule_kernel(float* __restrict__ o, const float* __restrict__ qn, const flo
   }
   if (n <= 0) return;
   const int kh = h / (heads / kv_heads);
-  const int i0 = kl * R;
-  const bool vec = (R % 4 == 0) && (dk % 4 == 0);
+  // rows kl, kl + 8, ...: the 8 lanes of a column read 8 consecutive LDS banks
   float* S = state + (((long)sl * heads + h) * dk) * dv;
   float st_[R];
   const bool fresh = pos0[s] <= 0;
 #pragma unroll
-  for (int r = 0; r < R; ++r) st_[r] = (!fresh && i0 + r < dk) ? S[(long)(i0 + r) * dv + c] : 0.f;
-  const long voff = 2L * kv_heads * dk + (long)h * dv + c;
-  float kk[R], qq[R], gg[R], nk[R], nq[R], ng[R];
-  float vv, bb, nv = 0.f, nb = 0.f;
-  {
-    const long row = r0;
-    load_rows<R>(nk, kn + (row * kv_heads + kh) * dk, i0, dk, vec);
-    load_rows<R>(nq, qn + (row * kv_heads + kh) * dk, i0, dk, vec);
-    load_rows<R>(ng, g + (row * heads + h) * dk, i0, dk, vec);
-    nv = ld(qkv, row * qkv_stride + voff);
-    nb = beta[row * heads + h];
-  }
-  for (int t = 0; t < n; ++t) {
-    const long row = r0 + t;
+  for (int r = 0; r < R; ++r) st_[r] = (!fresh && kl + kKL * r < dk) ? S[(long)(kl + kKL * r) * dv + c] : 0.f;
+  const long voff = 2L * kv_heads * dk + (long)h * dv + (long)blockIdx.x * kCols;
+
+  float ld_[P::NLD], lv_[P::NV], lb_ = 0.f;
+  // issue the global loads of the chunk that starts at row t0 (cnt rows)
+  auto fetch = [&](int t0, int cnt) {
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-      kk[r] = nk[r];
-      qq[r] = nq[r];
-      gg[r] = ng[r];
+    for (int u = 0; u < P::NLD; ++u) {
+      const int e = tid + 256 * u;                  // (row tt, array a, entry i) of the chunk
+      const int tt = e / (3 * P::DKP), rem = e % (3 * P::DKP);
+      const int a = rem / P::DKP, i = rem % P::DKP;
+      float v = 0.f;
+      if (tt < cnt && i < dk) {
+        const long row = r0 + t0 + tt;
+        v = a == 0 ? kn[(row * kv_heads + kh) * dk + i]
+          : a == 1 ? qn[(row * kv_heads + kh) * dk + i]
+                   : g[(row * heads + h) * dk + i];
+      }
+      ld_[u] = v;
     }
-    vv = nv;
-    bb = nb;
-    if (t + 1 < n) {
-      const long nx = row + 1;
-      load_rows<R>(nk, kn + (nx * kv_heads + kh) * dk, i0, dk, vec);
-      load_rows<R>(nq, qn + (nx * kv_heads + kh) * dk, i0, dk, vec);
-      load_rows<R>(ng, g + (nx * heads + h) * dk, i0, dk, vec);
-      nv = ld(qkv, nx * qkv_stride + voff);
-      nb = beta[nx * heads + h];
-    }
-    float dot = 0.f;
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-      st_[r] *= gg[r];
-      dot += st_[r] * kk[r];
+    for (int u = 0; u < P::NV; ++u) {
+      const int e = tid + 256 * u;
+      const int tt = e / kCols, cc = e % kCols;
+      lv_[u] = (tt < cnt && blockIdx.x * kCols + cc < dv)
+                   ? ld(qkv, (long)(r0 + t0 + tt) * qkv_stride + voff + cc) : 0.f;
     }
-    dot = sum8(dot);
-    const float u = bb * (vv - dot);
-    float out = 0.f;
+    lb_ = tid < cnt ? beta[(long)(r0 + t0 + tid) * heads + h] : 0.f;
+  };
+  auto park = [&](float* buf) {
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-      st_[r] += kk[r] * u;
-      out += st_[r] * qq[r];
+    for (int u = 0; u < P::NLD; ++u) {
+      const int e = tid + 256 * u;
+      const int tt = e / (3 * P::DKP), rem = e % (3 * P::DKP);
+      if (tt < P::TT) buf[tt * P::ROWF + rem] = ld_[u];
     }
-    out = sum8(out);
-    if (live && kl == 0) o[row * o_stride + (long)h * dv + col] = out;
+#pragma unroll
+    for (int u = 0; u < P::NV; ++u) {
+      const int e = tid + 256 * u;
+      if (e < P::TT * kCols) buf[(e / kCols) * P::ROWF + 3 * P::DKP + e % kCols] = lv_[u];
+    }
+    if (tid < P::TT) buf[tid * P::ROWF + 3 * P::DKP + kCols] = lb_;
+  };
+
+  fetch(0, min(P::TT, n));
+  park(stage[0]);
+  __syncthreads();
+  int cur = 0;
+  for (int t0 = 0; t0 < n; t0 += P::TT) {
+    const int cnt = min(P::TT, n - t0);
+    const bool more = t0 + P::TT < n;
+    if (more) fetch(t0 + P::TT, min(P::TT, n - t0 - P::TT));
+    const float* buf = stage[cur];
+    for (int t = 0; t < cnt; ++t) {
+      const float* rw = buf + t * P::ROWF;
+      float kk[R], qq[R];
+      float dot = 0.f;
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        kk[r] = rw[kl + kKL * r];
+        qq[r] = rw[P::DKP + kl + kKL * r];
+        st_[r] *= rw[2 * P::DKP + kl + kKL * r];
+        dot += st_[r] * kk[r];
+      }
+      dot = sum8(dot);
+      const float u = rw[3 * P::DKP + kCols] * (rw[3 * P::DKP + cl] - dot);
+      float out = 0.f;
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        st_[r] += kk[r] * u;
+        out += st_[r] * qq[r];
+      }
+      out = sum8(out);
+      if (live && kl == 0) o[(long)(r0 + t0 + t) * o_stride + (long)h * dv + col] = out;
+    }
+    if (more) park(stage[cur ^ 1]);
+    __syncthreads();
+    cur ^= 1;
   }
   if (live) {
 #pragma unroll
     for (int r = 0; r < R; ++r)
-      if (i0 + r < dk) S[(long)(i0 + r) * dv + col] = st_[r];
+      if (kl + kKL * r < dk) S[(long)(kl + kKL * r) * dv + col] = st_[r];
   }
 }
 

@@ -155,6 +155,22 @@ latent_attention_kernel(float* __restrict__ out, const float* __restrict__ qa, c
 // is read once per head group instead of once per head.  Each workgroup leaves (max,
 // sum, weighted c sums) per head; latent_combine_kernel merges the slices.
 // ---------------------------------------------------------------------------------
+// sum over the 16 lanes of a row (quad swaps, mirrored half row, mirrored row): every
+// lane gets the total
+__device__ __forceinline__ float sum16(float v) {
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, true));
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xF, 0xF, true));
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xF, 0xF, true));
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xF, 0xF, true));
+  return v;
+}
+
+constexpr int kSplitTK = 16;   // most keys per staged tile
+
+// 256 threads = 16 heads x 16 lanes.  The 16 lanes of a head split the dot products'
+// dimension (scores) and the rank axis (sums); scores are reduced over them on the lane
+// permute path, the softmax state (running max / sum) and the sums live in registers,
+// so the only barriers are those around staging a tile.  ACC = ceil(rank / 16).
 template <typename TC, int ACC>
 __global__ void __launch_bounds__(256)
 latent_split_kernel(float* __restrict__ ws_acc, float* __restrict__ ws_ml, const float* __restrict__ qa,
@@ -173,11 +189,9 @@ latent_split_kernel(float* __restrict__ ws_acc, float* __restrict__ ws_ml, const
   const int width = rank + dr, ldk = width | 1;   // odd strides: heads / keys land on different banks
   float* qs = smem;                       // [hg, ldk]
   float* kt = qs + hg * ldk;              // [tk, ldk]
-  float* ps = kt + tk * ldk;              // [hg, tk]
-  float* ms = ps + hg * tk;               // [hg] running max
-  float* ls = ms + hg;                    // [hg] running sum
-  float* al = ls + hg;                    // [hg] rescale of this tile
   const int tid = threadIdx.x;
+  const int hl = tid >> 4, ds = tid & 15;
+  const bool on = hl < nh;
   int nk = pos0[s] + rel + 1;
   if (nk > kv_len[s]) nk = kv_len[s];
   const int per = (nk + splits - 1) / splits;
@@ -187,15 +201,13 @@ latent_split_kernel(float* __restrict__ ws_acc, float* __restrict__ ws_ml, const
   for (int e = tid; e < nh * width; e += 256) {
     const int h = e / width, i = e % width;
     qs[h * ldk + i] = i < rank ? qa[((long)(h0 + h) * total_rows + row) * rank + i]
-                     : qr[(row * heads + h0 + h) * dr + (i - rank)];
+                               : qr[(row * heads + h0 + h) * dr + (i - rank)];
   }
-  if (tid < hg) {
-    ms[tid] = -INFINITY;
-    ls[tid] = 0.f;
-  }
+  float m = -INFINITY, l = 0.f;
   float acc[ACC];
 #pragma unroll
   for (int a = 0; a < ACC; ++a) acc[a] = 0.f;
+  const float* q = qs + (on ? hl : 0) * ldk;
   for (int k0 = k_begin; k0 < k_end; k0 += tk) {
     const int cnt = min(tk, k_end - k0);
     __syncthreads();                      // the previous tile is no longer read
@@ -207,54 +219,54 @@ latent_split_kernel(float* __restrict__ ws_acc, float* __restrict__ ws_ml, const
       kt[j * ldk + i] = ld(cache, ((long)blk * block_size + tok % block_size) * width + i);
     }
     __syncthreads();
-    for (int p = tid; p < nh * cnt; p += 256) {
-      const int h = p / cnt, j = p % cnt;
-      const float* q = qs + h * ldk;
-      const float* k = kt + j * ldk;
-      float d = 0.f;
-      for (int i = 0; i < width; ++i) d += q[i] * k[i];
-      ps[h * tk + j] = d * scale;
+    float p[kSplitTK];
+#pragma unroll
+    for (int j = 0; j < kSplitTK; ++j) p[j] = 0.f;
+    for (int i = ds; i < width; i += 16) {
+      const float qv = q[i];
+#pragma unroll
+      for (int j = 0; j < kSplitTK; ++j)
+        if (j < cnt) p[j] += qv * kt[j * ldk + i];
     }
-    __syncthreads();
-    if (tid < nh) {
-      float* pr = ps + tid * tk;
-      float mt = -INFINITY;
-      for (int j = 0; j < cnt; ++j) mt = fmaxf(mt, pr[j]);
-      const float mo = ms[tid], mn = fmaxf(mo, mt);
-      float sum = 0.f;
-      for (int j = 0; j < cnt; ++j) {
-        const float e = expf(pr[j] - mn);
-        pr[j] = e;
-        sum += e;
-      }
-      const float a = expf(mo - mn);      // 0 at the first tile (mo = -inf)
-      al[tid] = a;
-      ls[tid] = ls[tid] * a + sum;
-      ms[tid] = mn;
+    float mt = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < kSplitTK; ++j) {
+      p[j] = sum16(p[j]) * scale;
+      if (j < cnt) mt = fmaxf(mt, p[j]);
     }
-    __syncthreads();
+    const float mn = fmaxf(m, mt);
+    const float alpha = expf(m - mn);     // 0 at the first tile (m = -inf)
+    float sum = 0.f;
+#pragma unroll
+    for (int j = 0; j < kSplitTK; ++j) {
+      p[j] = j < cnt ? expf(p[j] - mn) : 0.f;
+      sum += p[j];
+    }
+    l = l * alpha + sum;
+    m = mn;
 #pragma unroll
     for (int a = 0; a < ACC; ++a) {
-      const int o = tid + 256 * a;
-      if (o < nh * rank) {
-        const int h = o / rank, d = o % rank;
-        float v = acc[a] * al[h];
-        const float* pr = ps + h * tk;
-        for (int j = 0; j < cnt; ++j) v += pr[j] * kt[j * ldk + d];
-        acc[a] = v;
+      const int d = ds + 16 * a;
+      float v = acc[a] * alpha;
+      if (d < rank) {
+#pragma unroll
+        for (int j = 0; j < kSplitTK; ++j)
+          if (j < cnt) v += p[j] * kt[j * ldk + d];
       }
+      acc[a] = v;
     }
   }
-  __syncthreads();
-  const long base = (row * splits + sp) * heads + h0;
+  if (on) {
+    const long base = (row * splits + sp) * heads + h0 + hl;
 #pragma unroll
-  for (int a = 0; a < ACC; ++a) {
-    const int o = tid + 256 * a;
-    if (o < nh * rank) ws_acc[(base + o / rank) * rank + o % rank] = acc[a];
-  }
-  if (tid < nh) {
-    ws_ml[(base + tid) * 2] = ms[tid];
-    ws_ml[(base + tid) * 2 + 1] = ls[tid];
+    for (int a = 0; a < ACC; ++a) {
+      const int d = ds + 16 * a;
+      if (d < rank) ws_acc[base * rank + d] = acc[a];
+    }
+    if (ds == 0) {
+      ws_ml[base * 2] = m;
+      ws_ml[base * 2 + 1] = l;
+    }
   }
 }
 
@@ -406,17 +418,16 @@ extern "C" int mx_latent_attention(float* out, const float* qa, const float* qr,
 // bytes, accumulators per thread (0: does not fit, use the per-row kernel)
 static int split_plan(int heads, int rank, int dr, int* hg, int* tk, size_t* lds) {
   const int width = rank + dr, ldk = width | 1;
-  int g = heads < 16 ? heads : 16;
-  while (g > 1 && (long)g * ldk > 9300) --g;
+  const int g = heads < 16 ? heads : 16;
   const long budget = 64 * 1024 / 4 - 64;
-  long t = (budget - (long)g * ldk - 3 * g) / (ldk + g);
+  long t = (budget - (long)g * ldk) / ldk;
   if (t < 2) return 0;
-  if (t > 32) t = 32;
-  const int acc = (g * rank + 255) / 256;
+  if (t > kSplitTK) t = kSplitTK;
+  const int acc = (rank + 15) / 16;
   if (acc > 64) return 0;
   *hg = g;
   *tk = (int)t;
-  *lds = (size_t)(g * ldk + t * ldk + g * t + 3 * g) * sizeof(float);
+  *lds = (size_t)(g * ldk + t * ldk) * sizeof(float);
   return acc;
 }
 
@@ -463,9 +474,7 @@ extern "C" int mx_latent_attention_split(float* out, float* ws_acc, float* ws_ml
                              bt_stride, heads, total_rows, rank, dr, block_size, num_blocks, scale,      \
                              skip_from, splits, hg, tk);                                                 \
   } while (0)
-  if (acc <= 1) MX_SPLIT(1);
-  else if (acc <= 2) MX_SPLIT(2);
-  else if (acc <= 4) MX_SPLIT(4);
+  if (acc <= 4) MX_SPLIT(4);
   else if (acc <= 8) MX_SPLIT(8);
   else if (acc <= 16) MX_SPLIT(16);
   else if (acc <= 32) MX_SPLIT(32);
