@@ -289,10 +289,10 @@ void latent_attention(Tensor out, Tensor qa, Tensor qr, Tensor cache, Tensor sta
   check_i32(bt, "block tables");
   TORCH_CHECK(bt.dim() == 2 && bt.size(0) >= num_segs && max_rows <= t, "block tables / max_rows");
   if (mx_latent_split_ws((int)heads, (int)rank, (int)dr)) {
-    // key slices: enough workgroups to fill the chip, at least ~64 keys per slice when
+    // key slices: enough workgroups to fill the chip (at most 16), at least ~64 keys per slice when
     // the longest context is known (max_kv; 0 inside captured graphs), scratch <= 256 MiB
     int64_t rows = std::max<int64_t>(1, std::min<int64_t>(t, num_segs * std::max<int64_t>(1, std::min(max_rows, skip_from > 0 ? skip_from - 1 : max_rows))));
-    int64_t splits = std::max<int64_t>(1, std::min<int64_t>(32, 512 / rows));
+    int64_t splits = std::max<int64_t>(1, std::min<int64_t>(16, 256 / rows));
     if (max_kv > 0) splits = std::max<int64_t>(1, std::min(splits, (max_kv + 63) / 64));
     while (splits > 1 && t * splits * heads * rank * 4 > (256LL << 20)) splits /= 2;
     auto f32 = qa.options();

@@ -167,6 +167,68 @@ __device__ __forceinline__ float sum16(float v) {
 
 constexpr int kSplitTK = 16;   // most keys per staged tile
 
+// Stages cnt <= 16 cache rows (keys k0..) into LDS as fp32, a wave per key: the wave's
+// keys' block-table entries and all their 16-byte loads are issued before anything is
+// stored, so one memory latency covers the tile.  Rows narrower than 16-byte groups, or
+// wider than 4 groups per lane, take the element-wise path.
+template <typename TC>
+__device__ __forceinline__ void stage_tile(float* __restrict__ kt, int ldk, const TC* __restrict__ cache,
+                                           const int* __restrict__ tab, int k0, int cnt, int width,
+                                           int block_size, int num_blocks, int wv, int lane) {
+  constexpr int VE = 16 / (int)sizeof(TC);          // elements per 16-byte group
+  constexpr int KW = kSplitTK / 4, CH = 4;          // keys per wave, groups per lane and key
+  const int groups = width / VE;
+  long base[KW];
+#pragma unroll
+  for (int u = 0; u < KW; ++u) {
+    const int j = wv + 4 * u;
+    base[u] = -1;
+    if (j < cnt) {
+      const int tok = k0 + j;
+      int blk = tab[tok / block_size];
+      if (blk < 0 || blk >= num_blocks) blk = 0;
+      base[u] = ((long)blk * block_size + tok % block_size) * width;
+    }
+  }
+  if (width % VE == 0 && groups <= 64 * CH) {
+    uint4 v[KW][CH];
+#pragma unroll
+    for (int u = 0; u < KW; ++u)
+#pragma unroll
+      for (int c = 0; c < CH; ++c) {
+        const int gidx = lane + 64 * c;
+        if (base[u] >= 0 && gidx < groups)
+          v[u][c] = *reinterpret_cast<const uint4*>(cache + base[u] + (long)gidx * VE);
+      }
+#pragma unroll
+    for (int u = 0; u < KW; ++u)
+#pragma unroll
+      for (int c = 0; c < CH; ++c) {
+        const int gidx = lane + 64 * c;
+        if (base[u] >= 0 && gidx < groups) {
+          float* dst = kt + (wv + 4 * u) * ldk + gidx * VE;
+          if constexpr (sizeof(TC) == 2) {
+            float f[8];
+            ft::load8(v[u][c], f);
+#pragma unroll
+            for (int k = 0; k < 8; ++k) dst[k] = f[k];
+          } else {
+            dst[0] = __uint_as_float(v[u][c].x);
+            dst[1] = __uint_as_float(v[u][c].y);
+            dst[2] = __uint_as_float(v[u][c].z);
+            dst[3] = __uint_as_float(v[u][c].w);
+          }
+        }
+      }
+  } else {
+#pragma unroll
+    for (int u = 0; u < KW; ++u)
+      if (base[u] >= 0)
+        for (int i = lane; i < width; i += 64) kt[(wv + 4 * u) * ldk + i] = ld(cache, base[u] + i);
+  }
+}
+
+
 // 256 threads = 16 heads x 16 lanes.  The 16 lanes of a head split the dot products'
 // dimension (scores) and the rank axis (sums); scores are reduced over them on the lane
 // permute path, the softmax state (running max / sum) and the sums live in registers,
@@ -198,10 +260,12 @@ latent_split_kernel(float* __restrict__ ws_acc, float* __restrict__ ws_ml, const
   const int chunk = (per + tk - 1) / tk * tk;
   const int k_begin = sp * chunk, k_end = min(nk, k_begin + chunk);
   const int* tab = bt + (long)s * bt_stride;
-  for (int e = tid; e < nh * width; e += 256) {
-    const int h = e / width, i = e % width;
-    qs[h * ldk + i] = i < rank ? qa[((long)(h0 + h) * total_rows + row) * rank + i]
-                               : qr[(row * heads + h0 + h) * dr + (i - rank)];
+  const int wv = tid >> 6, lane = tid & 63;
+  for (int h = wv; h < nh; h += 4) {      // a wave per head: independent coalesced loads
+    const float* qah = qa + ((long)(h0 + h) * total_rows + row) * rank;
+    const float* qrh = qr + (row * heads + h0 + h) * dr;
+    for (int i = lane; i < rank; i += 64) qs[h * ldk + i] = qah[i];
+    for (int i = lane; i < dr; i += 64) qs[h * ldk + rank + i] = qrh[i];
   }
   float m = -INFINITY, l = 0.f;
   float acc[ACC];
@@ -211,13 +275,7 @@ latent_split_kernel(float* __restrict__ ws_acc, float* __restrict__ ws_ml, const
   for (int k0 = k_begin; k0 < k_end; k0 += tk) {
     const int cnt = min(tk, k_end - k0);
     __syncthreads();                      // the previous tile is no longer read
-    for (int e = tid; e < cnt * width; e += 256) {
-      const int j = e / width, i = e % width;
-      const int tok = k0 + j;
-      int blk = tab[tok / block_size];
-      if (blk < 0 || blk >= num_blocks) blk = 0;
-      kt[j * ldk + i] = ld(cache, ((long)blk * block_size + tok % block_size) * width + i);
-    }
+    stage_tile<TC>(kt, ldk, cache, tab, k0, cnt, width, block_size, num_blocks, wv, lane);
     __syncthreads();
     float p[kSplitTK];
 #pragma unroll
@@ -280,19 +338,24 @@ __global__ void latent_combine_kernel(float* __restrict__ out, const float* __re
   if (rel >= n || (skip_from > 0 && n >= skip_from)) return;
   const long row = r0 + rel;
   const int h = blockIdx.z;
+  float M = -INFINITY;
+  for (int sp = 0; sp < splits; ++sp) M = fmaxf(M, ws_ml[((row * splits + sp) * heads + h) * 2]);
+  float L = 0.f;
+  for (int sp = 0; sp < splits; ++sp) {
+    const long b = (row * splits + sp) * heads + h;
+    const float m = ws_ml[b * 2];
+    L += m == -INFINITY ? 0.f : expf(m - M) * ws_ml[b * 2 + 1];
+  }
+  const float inv = L > 0.f ? 1.0f / L : 0.f;
   for (int d = threadIdx.x; d < rank; d += blockDim.x) {
-    float M = -INFINITY;
-    for (int sp = 0; sp < splits; ++sp) M = fmaxf(M, ws_ml[((row * splits + sp) * heads + h) * 2]);
-    float L = 0.f, v = 0.f;
+    float v = 0.f;
     for (int sp = 0; sp < splits; ++sp) {
       const long b = (row * splits + sp) * heads + h;
       const float m = ws_ml[b * 2];
-      if (m == -INFINITY) continue;       // an empty slice
-      const float w = expf(m - M);
-      L += w * ws_ml[b * 2 + 1];
+      const float w = m == -INFINITY ? 0.f : expf(m - M);   // an empty slice left zeros
       v += w * ws_acc[b * rank + d];
     }
-    out[((long)h * total_rows + row) * rank + d] = L > 0.f ? v / L : 0.f;
+    out[((long)h * total_rows + row) * rank + d] = v * inv;
   }
 }
 
