@@ -23,9 +23,7 @@ int mx_clamp_swiglu(void* out, const void* gu, int bf16, long gu_stride, long ro
 int mx_side_gate(void* out, const void* gpre, const void* table, int bf16, long table_stride, const int* ids,
                  int col0, long rows, int sd, int vocab, hipStream_t s);
 int mx_scale_add_rows(float* out, const void* y, int y_bf16, const int* rows, const void* weights, int w_bf16,
-                      long w_stride, int sigmoid, long n, int width, int out_rows, hipStream_t s);
-int mx_gather_combine(float* out, const void* y, int y_bf16, const int* src, const float* w, long rows, int top,
-                      int width, long y_rows, int accumulate, hipStream_t s);
+                      int sigmoid, long n, int width, int out_rows, hipStream_t s);
 int mx_short_conv_silu(void* out, const void* x, int bf16, const float* w, float* hist, const int* start,
                        const int* pos0, const int* slot, int num_segs, int max_rows, int channels, int taps,
                        int num_slots, hipStream_t s);
@@ -58,7 +56,7 @@ int mx_causal_softmax(void* P, int p_bf16, const float* S, long rows, int rows_p
                       float scale, hipStream_t s);
 int mx_moe_pairs(float* out, void* y, const void* h, int bf16, long h_stride, const int* idx, const float* wts,
                  const void* wgu, const void* wdown, long rows, int top, int experts, int ff, int width,
-                 float limit, int accumulate, hipStream_t s);
+                 float limit, hipStream_t s);
 int mx_moe_topk(int* idx, float* wts, const float* z, const float* corr, long rows, int experts, int top,
                 int groups, int keep, hipStream_t s);
 }
@@ -184,13 +182,13 @@ void scale_add_rows(Tensor out, Tensor y, OptT rows, Tensor weights, bool sigmoi
   check_f32(out, "out");
   TORCH_CHECK(y.is_cuda() && is_act(y) && y.is_contiguous() && y.dim() == 2 && out.dim() == 2 &&
               y.size(1) == out.size(1), "y");
-  TORCH_CHECK(weights.is_cuda() && is_act(weights) && weights.dim() == 1 && weights.numel() == y.size(0),
-              "weights: 1-D (any stride), one per row of y");
+  TORCH_CHECK(weights.is_cuda() && is_act(weights) && weights.is_contiguous() && weights.numel() == y.size(0),
+              "weights");
   if (rows) { check_i32(*rows, "rows"); TORCH_CHECK(rows->numel() == y.size(0), "rows size"); }
   else TORCH_CHECK(y.size(0) == out.size(0), "identity rows need equal row counts");
   chk(mx_scale_add_rows(out.data_ptr<float>(), y.data_ptr(), bf(y), rows ? rows->data_ptr<int>() : nullptr,
-                        weights.data_ptr(), bf(weights), weights.numel() ? weights.stride(0) : 1, sigmoid ? 1 : 0,
-                        y.size(0), (int)y.size(1), (int)out.size(0), stream()), "scale_add_rows");
+                        weights.data_ptr(), bf(weights), sigmoid ? 1 : 0, y.size(0), (int)y.size(1),
+                        (int)out.size(0), stream()), "scale_add_rows");
 }
 
 void short_conv_silu(Tensor out, Tensor x, Tensor w, Tensor hist, Tensor start, Tensor pos0, Tensor slot,
@@ -334,20 +332,7 @@ void moe_topk(Tensor idx, Tensor wts, Tensor z, Tensor corr, int64_t top, int64_
                   z.size(0), (int)z.size(1), (int)top, (int)groups, (int)keep, stream()), "moe_topk");
 }
 
-void gather_combine(Tensor out, Tensor y, Tensor src, Tensor w, bool accumulate) {
-  check_f32(out, "out");
-  check_i32(src, "src");
-  check_f32(w, "w");
-  TORCH_CHECK(y.is_cuda() && is_act(y) && y.is_contiguous() && y.dim() == 2 && out.dim() == 2 &&
-              y.size(1) == out.size(1) && src.dim() == 2 && src.size(0) == out.size(0) && w.sizes() == src.sizes(),
-              "gather_combine shapes");
-  chk(mx_gather_combine(out.data_ptr<float>(), y.data_ptr(), bf(y), src.data_ptr<int>(), w.data_ptr<float>(),
-                        out.size(0), (int)src.size(1), (int)out.size(1), y.size(0), accumulate ? 1 : 0, stream()),
-      "gather_combine");
-}
-
-void moe_pairs(Tensor out, Tensor h, Tensor idx, Tensor wts, Tensor wgu, Tensor wdown, double limit,
-               bool accumulate) {
+void moe_pairs(Tensor out, Tensor h, Tensor idx, Tensor wts, Tensor wgu, Tensor wdown, double limit) {
   check_f32(out, "out");
   check_rows(h, "h");
   check_i32(idx, "idx");
@@ -365,7 +350,7 @@ void moe_pairs(Tensor out, Tensor h, Tensor idx, Tensor wts, Tensor wgu, Tensor 
   Tensor y = at::empty({rows * top, ff}, h.options());
   chk(mx_moe_pairs(out.data_ptr<float>(), y.data_ptr(), h.data_ptr(), bf(h), h.stride(0), idx.data_ptr<int>(),
                    wts.data_ptr<float>(), wgu.data_ptr(), wdown.data_ptr(), rows, (int)top, (int)experts, (int)ff,
-                   (int)width, (float)limit, accumulate ? 1 : 0, stream()), "moe_pairs");
+                   (int)width, (float)limit, stream()), "moe_pairs");
 }
 
 }  // namespace
@@ -386,7 +371,6 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("causal_softmax", &causal_softmax);
   m.def("moe_topk", &moe_topk);
   m.def("moe_pairs", &moe_pairs);
-  m.def("gather_combine", &gather_combine);
   m.def("delta_max_dk", []() { return (int64_t)mx_delta_max_dk(); });
   m.def("latent_max_rank", []() { return (int64_t)mx_latent_max_rank(); });
 }

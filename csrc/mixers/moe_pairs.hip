@@ -2,7 +2,7 @@
 // back on the host): every (row, chosen expert) pair streams its expert's weights.
 //
 //   moe_gu_pairs:   y[pair, c] = glu(W_gate[e] h, W_up[e] h)[c]      (clamped GLU fused)
-//   moe_down_pairs: out[row, c] (= or +=) sum_k w[row, k] * (W_down[e_k] y[row, k])[c]   (fp32)
+//   moe_down_pairs: out[row, c] += sum_k w[row, k] * (W_down[e_k] y[row, k])[c]   (fp32)
 //
 // One wave per output column, lanes along the reduction axis with 16-byte loads where
 // the row length allows; the few rows' activations stay in L1/L2 while each expert
@@ -77,7 +77,7 @@ template <typename T>
 __global__ void __launch_bounds__(256)
 moe_down_pairs_kernel(float* __restrict__ out, const T* __restrict__ y, const int* __restrict__ idx,
                       const float* __restrict__ wts, const T* __restrict__ wdown, int top, int experts,
-                      int ff, int width, int vec, int accumulate) {
+                      int ff, int width, int vec) {
   const int row = blockIdx.y;
   const int c = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (c >= width) return;
@@ -92,7 +92,7 @@ moe_down_pairs_kernel(float* __restrict__ out, const T* __restrict__ y, const in
     st(tmp, 0, d);
     acc += wts[row * top + k] * ld(tmp, 0);
   }
-  if (lane == 0) out[(long)row * width + c] = accumulate ? out[(long)row * width + c] + acc : acc;
+  if (lane == 0) out[(long)row * width + c] += acc;
 }
 
 }  // namespace mx
@@ -101,7 +101,7 @@ using namespace mx;
 
 extern "C" int mx_moe_pairs(float* out, void* y, const void* h, int bf16, long h_stride, const int* idx,
                             const float* wts, const void* wgu, const void* wdown, long rows, int top,
-                            int experts, int ff, int width, float limit, int accumulate, hipStream_t s) {
+                            int experts, int ff, int width, float limit, hipStream_t s) {
   if (rows <= 0) return 0;
   const long pairs = rows * top;
   if (pairs > 65535 || rows > 65535) return -1;
@@ -113,6 +113,6 @@ extern "C" int mx_moe_pairs(float* out, void* y, const void* h, int bf16, long h
                                          width, limit, vec_gu));
   MX_DISPATCH_T(bf16, hipLaunchKernelGGL((moe_down_pairs_kernel<T>), dim3((width + 3) / 4, (unsigned)rows),
                                          dim3(256), 0, s, out, (const T*)y, idx, wts, (const T*)wdown, top,
-                                         experts, ff, width, vec_dn, accumulate));
+                                         experts, ff, width, vec_dn));
   return (int)hipGetLastError();
 }

@@ -124,45 +124,19 @@ __global__ void side_gate_kernel(T* __restrict__ out, const T* __restrict__ gpre
 template <typename TY, typename TW>
 __global__ void scale_add_rows_kernel(float* __restrict__ out, const TY* __restrict__ y,
                                       const int* __restrict__ rows, const TW* __restrict__ weights,
-                                      long w_stride, int sigmoid, int width, int out_rows) {
+                                      int sigmoid, int width, int out_rows) {
   const long i = blockIdx.x;
   const long dst = rows != nullptr ? rows[i] : i;
   if (dst < 0 || dst >= out_rows) return;
-  float w = ld(weights, i * w_stride);
+  float w = ld(weights, i);
   if (sigmoid) w = sigmoidf_(w);
   for (int c = threadIdx.x; c < width; c += blockDim.x)
     out[dst * width + c] += w * ld(y, i * width + c);
 }
 
-// out[t] (= or +=) sum_k w[t, k] * y[src[t, k]]: combines each row's expert outputs from
-// wherever the expert-sorted layout put them; one workgroup per row, no atomics
-template <typename TY>
-__global__ void gather_combine_kernel(float* __restrict__ out, const TY* __restrict__ y,
-                                      const int* __restrict__ src, const float* __restrict__ w, int top,
-                                      int width, long y_rows, int accumulate) {
-  const long t = blockIdx.x;
-  for (int c = threadIdx.x; c < width; c += blockDim.x) {
-    float acc = accumulate ? out[t * width + c] : 0.f;
-    for (int k = 0; k < top; ++k) {
-      long r = src[t * top + k];
-      if (r < 0 || r >= y_rows) continue;
-      acc += w[t * top + k] * ld(y, r * width + c);
-    }
-    out[t * width + c] = acc;
-  }
-}
-
 }  // namespace mx
 
 using namespace mx;
-
-extern "C" int mx_gather_combine(float* out, const void* y, int y_bf16, const int* src, const float* w,
-                                 long rows, int top, int width, long y_rows, int accumulate, hipStream_t s) {
-  if (rows <= 0) return 0;
-  MX_DISPATCH_T(y_bf16, hipLaunchKernelGGL((gather_combine_kernel<T>), dim3((unsigned)rows), dim3(256), 0, s, out,
-                                           (const T*)y, src, w, top, width, y_rows, accumulate));
-  return (int)hipGetLastError();
-}
 
 extern "C" int mx_embed_rows(float* out, const int* ids, const void* table, int bf16, int rows,
                              int width, int vocab, hipStream_t s) {
@@ -240,20 +214,20 @@ extern "C" int mx_side_gate(void* out, const void* gpre, const void* table, int 
 }
 
 extern "C" int mx_scale_add_rows(float* out, const void* y, int y_bf16, const int* rows,
-                                 const void* weights, int w_bf16, long w_stride, int sigmoid, long n,
-                                 int width, int out_rows, hipStream_t s) {
+                                 const void* weights, int w_bf16, int sigmoid, long n, int width,
+                                 int out_rows, hipStream_t s) {
   if (n <= 0) return 0;
   const dim3 grid((unsigned)n), block(256);
   if (y_bf16 && w_bf16)
     hipLaunchKernelGGL((scale_add_rows_kernel<bf16_t, bf16_t>), grid, block, 0, s, out, (const bf16_t*)y,
-                       rows, (const bf16_t*)weights, w_stride, sigmoid, width, out_rows);
+                       rows, (const bf16_t*)weights, sigmoid, width, out_rows);
   else if (y_bf16)
     hipLaunchKernelGGL((scale_add_rows_kernel<bf16_t, float>), grid, block, 0, s, out, (const bf16_t*)y,
-                       rows, (const float*)weights, w_stride, sigmoid, width, out_rows);
+                       rows, (const float*)weights, sigmoid, width, out_rows);
   else if (w_bf16)
     return -1;
   else
     hipLaunchKernelGGL((scale_add_rows_kernel<float, float>), grid, block, 0, s, out, (const float*)y,
-                       rows, (const float*)weights, w_stride, sigmoid, width, out_rows);
+                       rows, (const float*)weights, sigmoid, width, out_rows);
   return (int)hipGetLastError();
 }

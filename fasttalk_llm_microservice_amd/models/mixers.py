@@ -126,7 +126,7 @@ class ChannelDelta:
         lo = F.linear(h, self.wlo)
         a = F.linear(lo[:, :self.ra], self.wa2)
         gp = F.linear(lo[:, self.ra:self.ra + self.rg], self.wg2)
-        b = lo[:, self.ra + self.rg:]
+        b = lo[:, self.ra + self.rg:].contiguous()
         qkv = M.short_conv_silu(qkv, self.conv_w, s_conv, ctx.seg)
         o = M.gated_delta_rule(qkv, a, b, self.a_log, self.dt_bias, s_rec, ctx.seg, self.heads,
                                self.kvh, self.dk, self.dv)
@@ -164,7 +164,7 @@ class MoEFF:
             raise ValueError("expert groups do not fit the expert count")
         self.e, self.top, self.limit, self.groups, self.keep = experts, top, float(limit), groups, keep
         self.dtype = dtype
-        self.router_t = get("router").to(device, dtype).t().contiguous()        # [width, experts]
+        self.router = get("router").to(device, torch.float32).contiguous()
         self.correction = get("correction").to(device, torch.float32).contiguous()
         gus, downs = zip(*[_glu_weights(get, f"e{i}.", dtype, device) for i in range(experts)])
         self.wgu = torch.stack(gus).contiguous()       # [E, 2 ff, width]
@@ -177,33 +177,26 @@ class MoEFF:
 
     def __call__(self, h, ctx=None) -> torch.Tensor:
         t, width = h.shape
-        out = torch.empty(t, width, dtype=torch.float32, device=h.device)
-        # fp32 router logits: bf16 operands with fp32 accumulation and output are the
-        # same numbers as the widened product
-        z = M.mm_f32(h, self.router_t)
+        out = torch.zeros(t, width, dtype=torch.float32, device=h.device)
+        z = F.linear(h.float(), self.router)
         idx, wts = M.moe_topk(z, self.correction, self.top, self.groups, self.keep)
         if t <= self.PAIR_ROWS:
             # decode-size steps: per-pair weight streaming, nothing read back on the host
-            M.moe_pairs(out, h, idx, wts, self.wgu, self.wdown, self.limit, accumulate=False)
+            M.moe_pairs(out, h, idx, wts, self.wgu, self.wdown, self.limit)
             return self._shared(out, h)
-        # rows sorted by expert, every expert's group padded to the largest group: the
-        # experts run as two batched products over [experts, capacity, .]
-        e, top = self.e, self.top
         flat = idx.view(-1).long()
         order = torch.argsort(flat, stable=True)
-        counts = torch.bincount(flat, minlength=e)
-        cap = int(counts.max())                                   # host round trip (eager steps)
-        first = torch.cumsum(counts, 0) - counts                   # start of each group in sorted order
-        es = flat.index_select(0, order)
-        place = es * cap + (torch.arange(order.numel(), device=h.device) - first.index_select(0, es))
-        hp = torch.zeros(e * cap, width, dtype=h.dtype, device=h.device)
-        hp.index_copy_(0, place, h.index_select(0, order // top))
-        gu = torch.bmm(hp.view(e, cap, width), self.wgu.transpose(1, 2))
-        y = M.clamp_swiglu(gu.view(e * cap, gu.shape[2]), self.limit)
-        d = torch.bmm(y.view(e, cap, y.shape[1]), self.wdown.transpose(1, 2)).view(e * cap, width)
-        src = torch.empty(order.numel(), dtype=torch.int32, device=h.device)
-        src.index_copy_(0, order, place.int())                     # where each (row, k) pair's output sits
-        M.gather_combine(out, d, src.view(t, top), wts, accumulate=False)
+        counts = torch.bincount(flat, minlength=self.e).tolist()
+        rows = (order // self.top).int()
+        w = wts.view(-1).index_select(0, order)
+        hs = h.index_select(0, rows.long())
+        a = 0
+        for e, n in enumerate(counts):
+            if n == 0:
+                continue
+            y = M.clamp_swiglu(F.linear(hs[a:a + n], self.wgu[e]), self.limit)
+            M.scale_add_rows(out, F.linear(y, self.wdown[e]), rows[a:a + n], w[a:a + n])
+            a += n
         return self._shared(out, h)
 
     # rows up to which every (row, expert) pair streams its expert's weights (decode);
@@ -215,7 +208,7 @@ class MoEFF:
             wgu, wdown = self.shared
             gu = F.linear(h, wgu)
             y = M.clamp_swiglu(gu, self.shared_limit)
-            M.scale_add_rows(out, F.linear(y, wdown), None, gu[:, -1], sigmoid=True)
+            M.scale_add_rows(out, F.linear(y, wdown), None, gu[:, -1].contiguous(), sigmoid=True)
         return out
 
 

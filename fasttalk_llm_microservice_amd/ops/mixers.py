@@ -279,24 +279,14 @@ def moe_topk(z, correction, top: int, groups: int, keep: int):
     return ref.moe_topk(z, correction, top, groups, keep)
 
 
-def moe_pairs(out, h, idx, wts, wgu, wdown, limit: float, accumulate: bool = True):
-    """Few rows (decode): out (fp32, in place) (+)= sum_k wts[:, k] * expert_{idx[:, k]}(h),
+def moe_pairs(out, h, idx, wts, wgu, wdown, limit: float):
+    """Few rows (decode): out (fp32, in place) += sum_k wts[:, k] * expert_{idx[:, k]}(h),
     every (row, expert) pair streaming its expert's [gate | up] and down matrices; no
     host round trip, so the step can be captured in a hipGraph."""
     if out.is_cuda:
-        native_mixers().moe_pairs(out, h, idx, wts, wgu, wdown, float(limit), accumulate)
+        native_mixers().moe_pairs(out, h, idx, wts, wgu, wdown, float(limit))
     else:
-        if not accumulate:
-            out.zero_()
         ref.moe_pairs(out, h, idx, wts, wgu, wdown, limit)
-
-
-def gather_combine(out, y, src, w, accumulate: bool = False):
-    """out[t] (+)= sum_k w[t, k] * y[src[t, k]] (fp32 out; src < 0 skips)."""
-    if out.is_cuda:
-        native_mixers().gather_combine(out, y, src, w, accumulate)
-    else:
-        ref.gather_combine(out, y, src, w, accumulate)
 
 
 def clamp_swiglu(gu, limit: float):

@@ -189,14 +189,6 @@ def moe_pairs(out, h, idx, wts, wgu, wdown, limit):
             out[t] += wts[t, k] * F.linear(y, wdown[e])[0].float()
 
 
-def gather_combine(out, y, src, w, accumulate):
-    g = y.float()[src.long().clamp_min(0)] * (w * (src >= 0)).unsqueeze(-1)     # [T, top, width]
-    if accumulate:
-        out.add_(g.sum(1))
-    else:
-        out.copy_(g.sum(1))
-
-
 def clamp_swiglu(gu, limit, rows_scale=None):
     """gu [n, 2*ff (+1)] = [gate | up (| per-row gate logit)] -> y [n, ff]:
     g = min(gate, limit), u = clamp(up, +-limit), y = g * sigmoid(1.702 g) * (u + 1)."""
