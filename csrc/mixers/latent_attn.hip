@@ -165,9 +165,9 @@ __device__ __forceinline__ float sum16(float v) {
   return v;
 }
 
-constexpr int kSplitTK = 16;   // most keys per staged tile
+constexpr int kSplitTK = 8;    // keys per staged tile (compile time: the inner loops carry no branches)
 
-// Stages cnt <= 16 cache rows (keys k0..) into LDS as fp32, a wave per key: the wave's
+// Stages cnt <= kSplitTK cache rows (keys k0..) into LDS as fp32, a wave per key: the wave's
 // keys' block-table entries and all their 16-byte loads are issued before anything is
 // stored, so one memory latency covers the tile.  Rows narrower than 16-byte groups, or
 // wider than 4 groups per lane, take the element-wise path.
@@ -177,6 +177,11 @@ __device__ __forceinline__ void stage_tile(float* __restrict__ kt, int ldk, cons
                                            int block_size, int num_blocks, int wv, int lane) {
   constexpr int VE = 16 / (int)sizeof(TC);          // elements per 16-byte group
   constexpr int KW = kSplitTK / 4, CH = 4;          // keys per wave, groups per lane and key
+  // rows past the tile's last key read as zeros (their scores are masked afterwards)
+#pragma unroll
+  for (int u = 0; u < KW; ++u)
+    if (wv + 4 * u >= cnt)
+      for (int i = lane; i < width; i += 64) kt[(wv + 4 * u) * ldk + i] = 0.f;
   const int groups = width / VE;
   long base[KW];
 #pragma unroll
@@ -283,21 +288,20 @@ latent_split_kernel(float* __restrict__ ws_acc, float* __restrict__ ws_ml, const
     for (int i = ds; i < width; i += 16) {
       const float qv = q[i];
 #pragma unroll
-      for (int j = 0; j < kSplitTK; ++j)
-        if (j < cnt) p[j] += qv * kt[j * ldk + i];
+      for (int j = 0; j < kSplitTK; ++j) p[j] += qv * kt[j * ldk + i];
     }
     float mt = -INFINITY;
 #pragma unroll
     for (int j = 0; j < kSplitTK; ++j) {
-      p[j] = sum16(p[j]) * scale;
-      if (j < cnt) mt = fmaxf(mt, p[j]);
+      p[j] = j < cnt ? sum16(p[j]) * scale : -INFINITY;   // (the select follows the reduction)
+      mt = fmaxf(mt, p[j]);
     }
     const float mn = fmaxf(m, mt);
     const float alpha = expf(m - mn);     // 0 at the first tile (m = -inf)
     float sum = 0.f;
 #pragma unroll
     for (int j = 0; j < kSplitTK; ++j) {
-      p[j] = j < cnt ? expf(p[j] - mn) : 0.f;
+      p[j] = expf(p[j] - mn);             // exp(-inf) = 0 for the masked keys
       sum += p[j];
     }
     l = l * alpha + sum;
@@ -308,8 +312,7 @@ latent_split_kernel(float* __restrict__ ws_acc, float* __restrict__ ws_ml, const
       float v = acc[a] * alpha;
       if (d < rank) {
 #pragma unroll
-        for (int j = 0; j < kSplitTK; ++j)
-          if (j < cnt) v += p[j] * kt[j * ldk + d];
+        for (int j = 0; j < kSplitTK; ++j) v += p[j] * kt[j * ldk + d];
       }
       acc[a] = v;
     }
@@ -481,16 +484,15 @@ extern "C" int mx_latent_attention(float* out, const float* qa, const float* qr,
 // bytes, accumulators per thread (0: does not fit, use the per-row kernel)
 static int split_plan(int heads, int rank, int dr, int* hg, int* tk, size_t* lds) {
   const int width = rank + dr, ldk = width | 1;
-  const int g = heads < 16 ? heads : 16;
+  int g = heads < 16 ? heads : 16;
   const long budget = 64 * 1024 / 4 - 64;
-  long t = (budget - (long)g * ldk) / ldk;
-  if (t < 2) return 0;
-  if (t > kSplitTK) t = kSplitTK;
+  while (g > 1 && (long)(g + kSplitTK) * ldk > budget) --g;
+  if ((long)(g + kSplitTK) * ldk > budget) return 0;
   const int acc = (rank + 15) / 16;
   if (acc > 64) return 0;
   *hg = g;
-  *tk = (int)t;
-  *lds = (size_t)(g * ldk + t * ldk) * sizeof(float);
+  *tk = kSplitTK;
+  *lds = (size_t)(g + kSplitTK) * ldk * sizeof(float);
   return acc;
 }
 
