@@ -240,7 +240,9 @@ class ModelRunner:
         # is handed against the tensors of the launch (this pool's blocks, the rotary
         # table's rows, the vocab) and reports into this word, read after each step
         self.d_check: Optional[torch.Tensor] = None
-        if self.is_gpu and getattr(ops.native(), "kernel_checks", False):
+        # (the Llama kernel extension is not touched for models that do not use it, so a
+        # checkout that only serves those builds only their kernels)
+        if self.is_gpu and not self.stateful and getattr(ops.native(), "kernel_checks", False):
             self.d_check = torch.zeros(4, dtype=torch.int32, device=self.device)
             ops.native().set_kernel_checks(self.d_check)
             log.warning("FT_KERNEL_CHECKS: bounds-checked kernels (KV pool %d blocks x %d, "
