@@ -821,6 +821,7 @@ class LLMEngine:
             raise EngineError("replay_step with queued steps")
         sched = self.scheduler
         items = []
+        entries = [e for e in entries if len(e[1]) > 0]     # an entry without tokens runs nothing
         for rid, toks, _ in entries:
             seq = sched.by_id.get(rid)
             if seq is None:

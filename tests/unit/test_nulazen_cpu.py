@@ -73,3 +73,25 @@ def test_state_slots_gate_admission(tmp_path):
     outs = eng.generate(prompts, SamplingParams(temperature=0.0, max_tokens=5, ignore_eos=True))
     assert [len(o) for o in outs] == [5] * 5
     assert eng.scheduler.slots.num_free() == 2 and eng.bm.num_free() == 8
+
+
+def test_replay_order_and_idle_steps(tmp_path):
+    """Wanted rows come back in the caller's order whatever the step's row order is; a
+    request may sit out a step; an entry without tokens and a step without entries run
+    nothing; a finished request's id can be used again."""
+    import numpy as np
+
+    d, cfg, P = C.make_model("b", 3, tmp_path)
+    eng = C.make_engine(d, "cpu", seqs=2, pages=8)
+    ta, tb = C.tokens(9, cfg["vocab"], 1), C.tokens(6, cfg["vocab"], 2)
+    wa, wb = C.oracle(cfg, P, ta), C.oracle(cfg, P, tb)
+    eng.replay_step([("a", ta[:4], [3, 0])])
+    lg = eng.replay_step([("a", ta[4:5], [0]), ("b", tb[:5], [4, 1, 2])])          # a decodes beside b's prompt
+    np.testing.assert_allclose(lg, np.stack([wa[4], wb[4], wb[1], wb[2]]), rtol=2e-4, atol=3e-4)
+    assert eng.replay_step([("a", [], [])]).shape == (0, cfg["vocab"])
+    assert eng.replay_step([], []).shape[0] == 0
+    lg = eng.replay_step([("b", tb[5:], [0])], end=["b"])                          # a sits this step out
+    np.testing.assert_allclose(lg[0], wb[5], rtol=2e-4, atol=3e-4)
+    lg = eng.replay_step([("b", tb[:2], [1]), ("a", ta[5:], [3])], end=["a", "b"])  # a new request named b
+    np.testing.assert_allclose(lg, np.stack([wb[1], wa[8]]), rtol=2e-4, atol=3e-4)
+    assert eng.scheduler.slots.num_free() == 2 and eng.bm.num_free() == 8
