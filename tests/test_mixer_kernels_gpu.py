@@ -130,10 +130,11 @@ def test_short_conv_segments(dt, taps):
 
 
 @pytest.mark.parametrize("dt", DTYPES)
-@pytest.mark.parametrize("heads,kvh,dk,dv", [(4, 2, 16, 24), (2, 2, 64, 64), (3, 1, 40, 33), (2, 1, 128, 128)])
+@pytest.mark.parametrize("heads,kvh,dk,dv", [(4, 2, 16, 24), (2, 2, 64, 64), (3, 1, 40, 33), (2, 1, 128, 128),
+                                             (2, 1, 200, 40), (1, 1, 3, 70)])
 def test_gated_delta_rule(dt, heads, kvh, dk, dv):
     g = torch.Generator().manual_seed(4)
-    lens, pos0, slots = [1, 6, 2, 1], [5, 0, 3, 0], [1, 0, -1, 2]
+    lens, pos0, slots = [1, 37, 2, 1], [5, 0, 3, 0], [1, 0, -1, 2]   # 37 rows: several staged chunks
     seg, _ = make_seg(lens, pos0, slots)
     t = sum(lens)
     qkv = rnd(t, 2 * kvh * dk + heads * dv, dt=dt, g=g)
@@ -151,7 +152,9 @@ def test_gated_delta_rule(dt, heads, kvh, dk, dv):
 
 
 @pytest.mark.parametrize("dt", DTYPES)
-@pytest.mark.parametrize("heads,dn,dr,rank,dims", [(3, 16, 8, 40, 8), (2, 32, 16, 64, 8), (5, 8, 4, 130, 4)])
+# (also: more than 16 heads -> several head groups; a wide row -> the head group shrinks to fit LDS)
+@pytest.mark.parametrize("heads,dn,dr,rank,dims", [(3, 16, 8, 40, 8), (2, 32, 16, 64, 8), (5, 8, 4, 130, 4),
+                                                    (20, 8, 4, 24, 4), (12, 8, 100, 900, 6)])
 def test_latent_attention_paged(dt, heads, dn, dr, rank, dims):
     g = torch.Generator().manual_seed(5)
     bs = 4
