@@ -1,6 +1,13 @@
 """Reusable sublayers built on :mod:`fasttalk_llm_microservice_amd.ops.mixers`:
-latent attention (paged latent cache), the channel-decay gated delta rule (state
-slots), dense and mixture-of-experts feed-forwards and the per-layer token-side input.
+latent attention (paged latent cache), windowed attention with sigmoid weights and
+windowed differential attention (paged key / value caches), the channel-decay gated
+delta rule and the selective state-space mixer (state slots), dense, gated and
+mixture-of-experts feed-forwards and the per-layer token-side input.
+
+Every mixer owns its cache layout: ``alloc_cache(num_blocks, block_size, dtype,
+num_slots, device)`` returns what its ``__call__`` takes as ``cache`` (pages indexed by
+the engine's block tables, or per-sequence state slots), and ``cache_bytes_per_token``
+what a token costs in pages.
 
 Each class takes its sizes and constants as constructor arguments and a ``get(name)``
 callable that returns a weight tensor ([out, in] for projections), so a model file only
@@ -29,6 +36,11 @@ class StepContext:
         self.positions = positions
         self.slot_mapping = slot_mapping
         self.seg = seg
+
+
+def _state_slots(shapes, num_slots: int, device):
+    """(recurrent state, convolution history) fp32, one row per state slot."""
+    return tuple(torch.zeros((num_slots,) + tuple(sh), dtype=torch.float32, device=device) for sh in shapes)
 
 
 class LatentAttention:
@@ -64,6 +76,12 @@ class LatentAttention:
 
     def cache_width(self) -> int:
         return self.rank + self.dr
+
+    def cache_bytes_per_token(self, elem_bytes: int) -> int:
+        return self.cache_width() * elem_bytes
+
+    def alloc_cache(self, num_blocks, block_size, dtype, num_slots, device):
+        return torch.zeros(num_blocks, block_size, self.cache_width(), dtype=dtype, device=device)
 
     def __call__(self, h, ctx: StepContext, cache) -> torch.Tensor:
         t = h.shape[0]
@@ -120,6 +138,12 @@ class ChannelDelta:
     def state_shapes(self):
         return (self.heads, self.dk, self.dv), (max(self.taps - 1, 0), self.channels)
 
+    def cache_bytes_per_token(self, elem_bytes: int) -> int:
+        return 0
+
+    def alloc_cache(self, num_blocks, block_size, dtype, num_slots, device):
+        return _state_slots(self.state_shapes(), num_slots, device)
+
     def __call__(self, h, ctx: StepContext, state) -> torch.Tensor:
         s_rec, s_conv = state
         qkv = F.linear(h, self.wqkv)
@@ -132,6 +156,167 @@ class ChannelDelta:
                                self.kvh, self.dk, self.dv)
         y = M.head_rms_gate(o, self.norm, gp, self.eps, self.heads, self.dv, self.dtype)
         return F.linear(y, self.wo)
+
+
+class WindowedAttention:
+    """Grouped-query attention over a sliding window of a paged key cache and a paged
+    value cache (common part of :class:`SigmoidAttention` and
+    :class:`DifferentialAttention`): the fused q|k|v(|extra) projection, the cache
+    layout and the choice between the per-row kernel (decode rows, short segments) and
+    banded matrix products (prefill chunks)."""
+
+    # segments of this many rows or more run as banded products
+    PRODUCT_ROWS = 32
+
+    def __init__(self, spec: M.WindowSpec, wqkv: torch.Tensor, bias: Optional[torch.Tensor],
+                 wo: torch.Tensor, eps: float, dtype):
+        sp = spec
+        if sp.heads % sp.kv_heads:
+            raise ValueError("heads must be a multiple of kv_heads")
+        self.spec, self.eps, self.dtype = spec, eps, dtype
+        self.nq = sp.heads * sp.maps * sp.dk
+        self.nk = sp.kv_heads * sp.maps * sp.dk
+        self.nv = sp.kv_heads * sp.dv
+        if wqkv.shape[0] < self.nq + self.nk + self.nv or wo.shape[1] != sp.heads * sp.dv:
+            raise ValueError("attention projections do not fit the head sizes")
+        self.wqkv, self.bias, self.wo = wqkv, bias, wo
+
+    def cache_bytes_per_token(self, elem_bytes: int) -> int:
+        return (self.nk + self.nv) * elem_bytes
+
+    def alloc_cache(self, num_blocks, block_size, dtype, num_slots, device):
+        return (torch.zeros(num_blocks, block_size, self.nk, dtype=dtype, device=device),
+                torch.zeros(num_blocks, block_size, self.nv, dtype=dtype, device=device))
+
+    def attend(self, q, ctx: StepContext, cache) -> torch.Tensor:
+        """fp32 [T, heads*maps, dv] for fp32 queries [T, heads*maps*dk]."""
+        kc, vc = cache
+        seg = ctx.seg
+        if seg.host is not None and seg.max_rows >= self.PRODUCT_ROWS:
+            out = torch.zeros(q.shape[0], self.spec.heads * self.spec.maps, self.spec.dv,
+                              dtype=torch.float32, device=q.device)
+            if min(b - a for a, b in zip(seg.host[0][:-1], seg.host[0][1:])) < self.PRODUCT_ROWS:
+                M.window_attention(q, kc, vc, seg, self.spec, skip_from=self.PRODUCT_ROWS, out=out)
+            return M.window_attention_products(out, q, kc, vc, seg, self.spec, self.PRODUCT_ROWS)
+        return M.window_attention(q, kc, vc, seg, self.spec)
+
+
+class SigmoidAttention(WindowedAttention):
+    """Windowed attention without softmax: q, k, v projections with biases, an RMS norm
+    over the whole q projection and over the whole k projection (weights of that size),
+    no rotation; a key's weight is sigmoid(q.k * scale - r1_h ln(1 + r2_h (i - j)) + pb_h),
+    not normalised over keys."""
+
+    def __init__(self, get: Get, width: int, heads: int, kv_heads: int, dim: int, vdim: int,
+                 window: int, scale: float, eps: float, dtype, device):
+        f32 = lambda n: get(n).to(device, torch.float32).contiguous()   # noqa: E731
+        spec = M.WindowSpec(heads, kv_heads, dim, vdim, int(window), float(scale), maps=1, sigmoid=True,
+                            r1=f32("r1"), r2=f32("r2"), pb=f32("pb"))
+        wqkv = torch.cat([get("q"), get("k"), get("v")], 0).to(device, dtype).contiguous()
+        bias = torch.cat([get("q.b"), get("k.b"), get("v.b")], 0).to(device, dtype).contiguous()
+        super().__init__(spec, wqkv, bias, get("o").to(device, dtype).contiguous(), eps, dtype)
+        self.q_norm, self.k_norm = f32("q.norm"), f32("k.norm")
+        if self.q_norm.numel() != self.nq or self.k_norm.numel() != self.nk or spec.r1.numel() != heads:
+            raise ValueError("attention norm / bias tensors do not fit the head sizes")
+
+    def __call__(self, h, ctx: StepContext, cache) -> torch.Tensor:
+        qkv = F.linear(h, self.wqkv, self.bias)
+        q = M.attn_prep(qkv, self.nq, self.nk, self.q_norm, self.k_norm, self.eps, None, 0, self.spec.dk,
+                        ctx.positions, ctx.slot_mapping, cache[0], cache[1])
+        o = self.attend(q, ctx, cache)
+        return F.linear(o.view(h.shape[0], -1).to(self.dtype), self.wo)
+
+
+class DifferentialAttention(WindowedAttention):
+    """Windowed differential attention: two softmax score maps per head ([map 1, map 2]
+    rows of q and k, head by head) over the same values, o = a1 - lam a2 with
+    lam = exp(lq1.lk1) - exp(lq2.lk2) + diff, o divided by its root mean square per head,
+    times (1 - diff), times a per-head sigmoid gate of the mixer's input.  Rotary
+    positions on the first ``rot_dims`` entries of every map (optionally with
+    wavelength-dependent frequency scaling)."""
+
+    def __init__(self, get: Get, width: int, heads: int, kv_heads: int, dim: int, vdim: int,
+                 window: int, scale: float, diff: float, rot_dims: int, rot_base: float, rot_scaling,
+                 eps: float, dtype, device, max_pos: int):
+        spec = M.WindowSpec(heads, kv_heads, dim, vdim, int(window), float(scale), maps=2)
+        # the gate's rows ride on the fused projection
+        wqkv = torch.cat([get("q"), get("k"), get("v"), get("g")], 0).to(device, dtype).contiguous()
+        super().__init__(spec, wqkv, None, get("o").to(device, dtype).contiguous(), eps, dtype)
+        if rot_dims % 2 or rot_dims > dim or wqkv.shape[0] != self.nq + self.nk + self.nv + heads:
+            raise ValueError("differential attention sizes do not fit")
+        f = lambda n: get(n).to(torch.float32).cpu()   # noqa: E731
+        self.diff = float(diff)
+        self.lam = float(torch.exp((f("lq1") * f("lk1")).sum()) - torch.exp((f("lq2") * f("lk2")).sum())
+                         + torch.tensor(self.diff, dtype=torch.float32))
+        self.rot_dims = int(rot_dims)
+        self.table = M.rope_table(max_pos, rot_dims, rot_base, device=device, scaling=rot_scaling) \
+            if rot_dims else None
+
+    def __call__(self, h, ctx: StepContext, cache) -> torch.Tensor:
+        qkvg = F.linear(h, self.wqkv)
+        n = self.nq + self.nk + self.nv
+        q = M.attn_prep(qkvg[:, :n], self.nq, self.nk, None, None, self.eps, self.table, self.rot_dims,
+                        self.spec.dk, ctx.positions, ctx.slot_mapping, cache[0], cache[1])
+        a = self.attend(q, ctx, cache)
+        o = M.diff_combine(a, qkvg[:, n:], self.lam, 1.0 - self.diff, self.eps, self.spec.heads,
+                           self.spec.dv, self.dtype)
+        return F.linear(o, self.wo)
+
+
+class StateSpaceMixer:
+    """Selective state-space mixer with a scalar decay per head (state-space duality
+    form): one input projection [z | x | B | C | dt], a short causal convolution with
+    bias and SiLU over x|B|C, the recurrence S <- exp(-exp(A) dt) S + dt B x^T,
+    y = S^T C + D x with dt = softplus(dt + dt_bias), then y silu(z), an RMS norm in
+    ``norm_groups`` equal parts with a weight, and the output projection."""
+
+    def __init__(self, get: Get, width: int, heads: int, vdim: int, state: int, groups: int, taps: int,
+                 norm_groups: int, eps: float, dtype, device):
+        self.heads, self.dv, self.n, self.groups, self.taps = heads, vdim, state, groups, taps
+        self.norm_groups, self.eps, self.dtype = norm_groups, eps, dtype
+        self.inner = heads * vdim
+        self.channels = self.inner + 2 * groups * state
+        if heads % groups or self.inner % norm_groups:
+            raise ValueError("state-space heads / groups do not divide")
+        f32 = lambda n: get(n).to(device, torch.float32).contiguous()   # noqa: E731
+        self.win = get("in").to(device, dtype).contiguous()
+        if self.win.shape[0] != self.inner + self.channels + heads:
+            raise ValueError("state-space input projection does not fit its sizes")
+        self.conv_w, self.conv_b = f32("conv"), f32("conv.b")
+        if self.conv_w.shape != (self.channels, taps):
+            raise ValueError("convolution weights do not fit the projection")
+        self.a_log, self.dt_bias, self.d_skip, self.norm = f32("A_log"), f32("dt_bias"), f32("D"), f32("norm")
+        self.wo = get("o").to(device, dtype).contiguous()
+
+    def state_shapes(self):
+        return (self.heads, self.n, self.dv), (max(self.taps - 1, 0), self.channels)
+
+    def cache_bytes_per_token(self, elem_bytes: int) -> int:
+        return 0
+
+    def alloc_cache(self, num_blocks, block_size, dtype, num_slots, device):
+        return _state_slots(self.state_shapes(), num_slots, device)
+
+    def __call__(self, h, ctx: StepContext, state) -> torch.Tensor:
+        s_rec, s_conv = state
+        p = F.linear(h, self.win)
+        z = p[:, :self.inner]
+        xbc = M.short_conv_silu(p[:, self.inner:self.inner + self.channels], self.conv_w, s_conv, ctx.seg,
+                                bias=self.conv_b)
+        y = M.ssd_scan(xbc, p[:, self.inner + self.channels:], self.a_log, self.dt_bias, self.d_skip, s_rec,
+                       ctx.seg, self.heads, self.groups, self.n, self.dv)
+        y = M.gate_group_norm(y, z, self.norm, self.eps, self.norm_groups, self.dtype)
+        return F.linear(y, self.wo)
+
+
+class GatedFF:
+    """down(gelu_tanh(gate h) * (up h))."""
+
+    def __init__(self, get: Get, dtype, device):
+        self.wgu, self.down = _glu_weights(get, "", dtype, device)
+
+    def __call__(self, h, ctx=None) -> torch.Tensor:
+        return F.linear(M.gelu_glu(F.linear(h, self.wgu)), self.down)
 
 
 class DenseFF:

@@ -23,13 +23,11 @@ import os
 from typing import Dict, List, Optional, Tuple
 
 import torch
-import torch.nn.functional as F
 
-from ..ops import mixers as M
 from ..parallel.comm import SINGLE, TPComm
-from . import weights as W
-from .mixers import ChannelDelta, DenseFF, LatentAttention, MoEFF, StepContext, TokenSide
+from .mixers import ChannelDelta, DenseFF, LatentAttention, MoEFF, TokenSide
 from .registry import Architecture, register
+from .stacked import StackedCache, StackedLayer, StackedModel
 
 log = logging.getLogger(__name__)
 
@@ -198,72 +196,27 @@ def save_checkpoint(cfg: NulazenConfig, tensors: Dict[str, torch.Tensor], out_di
         json.dump(config_to_dict(cfg), f, indent=1)
 
 
-@dataclasses.dataclass
-class _Layer:
-    kind: str
-    norm1: torch.Tensor
-    norm1b: torch.Tensor
-    mixer: object
-    norm2: Optional[torch.Tensor] = None
-    norm2b: Optional[torch.Tensor] = None
-    ff: Optional[object] = None
-    side: Optional[TokenSide] = None
+_Layer = StackedLayer
+NulazenCache = StackedCache
 
 
-class NulazenCache:
-    """Per layer run: a paged latent cache [num_blocks, block_size, rank + rot_dim]
-    (latent-attention runs) or (recurrent state [slots, heads, dk, dv] fp32, convolution
-    history [slots, taps-1, channels] fp32) (delta-rule runs)."""
-
-    def __init__(self, per_run: list):
-        self.per_run = per_run
-
-    def tensors(self):
-        for c in self.per_run:
-            yield from ((c,) if isinstance(c, torch.Tensor) else c)
-
-
-class NulazenModel:
-    needs_state_slots = True     # the runner hands every sequence a state slot
+class NulazenModel(StackedModel):
+    family = "Nulazen"
     # decode steps up to this many rows run without a host round trip (per-pair expert
     # kernels) and are captured in hipGraphs; larger steps sort rows by expert on the host
-    supports_graphs = True
     max_graph_rows = MoEFF.PAIR_ROWS
 
     def __init__(self, cfg: NulazenConfig, device, dtype=torch.bfloat16, comm: TPComm = SINGLE,
                  max_model_len: int = 8192, quantization: Optional[str] = None):
-        if comm.world_size != 1:
-            raise ValueError("Nulazen runs on one device (tensor parallelism is not implemented)")
-        if quantization:
-            raise ValueError("Nulazen has no quantized weight path")
-        self.cfg, self.device, self.dtype, self.comm = cfg, torch.device(device), dtype, comm
-        self.tp, self.rank = 1, 0
-        self.max_model_len = max_model_len
-        self.runs = cfg.runs()
-        self.layers: List[_Layer] = []
-        self.embed = self.head = self.final_norm = self.loop_step = self.side_embed = None
-        self.mark_at = None
-        self.layer_tap: Optional[list] = None   # tests: fp32 residual after every layer run
-        self.invariant = False
-        self._mm_out_dtype = True
-        if self.device.type == "cuda":
-            # true fp32 / fp32-accumulated products from the vendor library
-            torch.backends.cuda.matmul.allow_tf32 = False
-            torch.backends.cuda.matmul.allow_bf16_reduced_precision_reduction = False
+        super().__init__(cfg, device, dtype, comm, max_model_len, quantization)
+        self.side_embed = None
 
     # ------------------------------------------------------------------ weights
     def load_tensors(self, get, has=lambda n: True):
         cfg, dev, dt = self.cfg, self.device, self.dtype
         eps = cfg.rms_norm_eps
         f32 = lambda n: get(n).to(dev, torch.float32)   # noqa: E731
-        self.embed = get("embed").to(dev, dt).contiguous()
-        head = get("head").to(dev, dt)
-        # the sampler reads logits rows in groups of 8: zero rows pad the head, and their
-        # logits are set to -inf (never sampled; callers that want logits cut them off)
-        self.vocab_pad = (-head.shape[0]) % 8
-        if self.vocab_pad:
-            head = torch.cat([head, torch.zeros(self.vocab_pad, head.shape[1], dtype=dt, device=dev)], 0)
-        self.head = head.contiguous()
+        self.load_head(get)
         self.final_norm = f32("final.norm")
         self.loop_step = f32("loop.step") if cfg.loop else None
         self.side_embed = get("side.embed").to(dev, dt).contiguous() if cfg.side_dim else None
@@ -281,7 +234,7 @@ class NulazenModel:
             else:
                 mixer = ChannelDelta(mget, cfg.hidden_size, m["heads"], m.get("kv_heads", m["heads"]),
                                      m["dim"], m["vdim"], m["conv"], eps, dt, dev)
-            L = _Layer(l["type"], f32(p + "norm1"), f32(p + "norm1b"), mixer)
+            L = StackedLayer(l["type"], f32(p + "norm1"), f32(p + "norm1b"), mixer)
             mlp = l["mlp"]
             if mlp is not None:
                 fget = lambda n, p=p: get(p + "mlp." + n)   # noqa: E731
@@ -301,120 +254,8 @@ class NulazenModel:
             self.layers.append(L)
         return self
 
-    def load_checkpoint(self, ckpt_dir: str):
-        idx = W.SafetensorsIndex(ckpt_dir)
-        return self.load_tensors(idx.get, idx.has)
-
-    def init_random(self, seed: int = 0, **_):
-        on = self.device if self.device.type == "cuda" else "cpu"
-        t = random_tensors(self.cfg, seed, torch.bfloat16, device=on)
-        return self.load_tensors(t.__getitem__)
-
-    def resident_weight_bytes(self) -> int:
-        seen, total = set(), 0
-        stack = [self.__dict__]
-        while stack:
-            o = stack.pop()
-            vals = o.values() if isinstance(o, dict) else o if isinstance(o, (list, tuple)) else \
-                vars(o).values() if hasattr(o, "__dict__") else ()
-            for v in vals:
-                if isinstance(v, torch.Tensor):
-                    if v.data_ptr() not in seen:
-                        seen.add(v.data_ptr())
-                        total += v.numel() * v.element_size()
-                elif isinstance(v, (dict, list, tuple)) or hasattr(v, "__dict__") and \
-                        type(v).__module__.startswith(__package__):
-                    stack.append(v)
-        return total
-
-    # ------------------------------------------------------------------ cache / state
-    def kv_block_bytes(self, block_size: int, dtype) -> int:
-        es = torch.tensor([], dtype=dtype).element_size()
-        return max(1, self.cfg.kv_bytes_per_token(es) * block_size)
-
-    def allocate_kv_cache(self, num_blocks: int, block_size: int, dtype=None, num_slots: int = 1):
-        """One cache / state per layer RUN (a looped layer owns one per pass)."""
-        dt = dtype or self.dtype
-        if dt not in (torch.float32, torch.bfloat16):
-            raise ValueError("the latent cache is kept in the compute dtype")
-        per_run = []
-        for i, _ in self.runs:
-            mx = self.layers[i].mixer
-            if isinstance(mx, LatentAttention):
-                per_run.append(torch.zeros(num_blocks, block_size, mx.cache_width(), dtype=dt,
-                                           device=self.device))
-            else:
-                s, c = mx.state_shapes()
-                per_run.append((torch.zeros((num_slots,) + s, dtype=torch.float32, device=self.device),
-                                torch.zeros((num_slots,) + c, dtype=torch.float32, device=self.device)))
-        return NulazenCache(per_run)
-
-    # ------------------------------------------------------------------ forward
-    def forward(self, input_ids: torch.Tensor, meta, caches: NulazenCache) -> torch.Tensor:
-        """Final-normed hidden rows (compute dtype) at ``meta.logits_indices``."""
-        cfg, dt, eps = self.cfg, self.dtype, self.cfg.rms_norm_eps
-        seg = meta.segments
-        if seg is None:
-            raise ValueError("Nulazen needs the step's row segments (AttnMeta.segments)")
-        ctx = StepContext(input_ids, meta.positions, meta.slot_mapping, seg)
-        x = M.embed_rows(input_ids, self.embed)
-        tap = self.layer_tap
-        fuse_step = tap is None
-        h = None
-        nruns = len(self.runs)
-        mark = self.mark_at
-        for r, (li, step) in enumerate(self.runs):
-            if mark is not None and r == mark[0]:
-                mark[1].record()
-            L = self.layers[li]
-            if h is None:   # first run, or the step vector was not fused into the last kernel
-                vec = self.loop_step[step] if step is not None and (r == 0 or not fuse_step) else None
-                h = M.rms_norm_rows(x, L.norm1, eps, dt, add_vec=vec)
-            y = L.mixer(h, ctx, caches.per_run[r])
-            nxt = self.runs[r + 1] if r + 1 < nruns else None
-            nvec = self.loop_step[nxt[1]] if nxt is not None and nxt[1] is not None and fuse_step else None
-            nw = self.layers[nxt[0]].norm1 if nxt is not None and (fuse_step or nxt[1] is None) else None
-            last = L.ff is None and L.side is None
-            h, xc = M.add_rms_norm_rows(x, y, L.norm1b, eps,
-                                        add_vec=nvec if last else None,
-                                        next_w=L.norm2 if L.ff is not None else (nw if last else None),
-                                        out_dtype=dt, want_cast=L.ff is None and L.side is not None)
-            if L.ff is not None:
-                y = L.ff(h, ctx)
-                last = L.side is None
-                h, xc = M.add_rms_norm_rows(x, y, L.norm2b, eps, add_vec=nvec if last else None,
-                                            next_w=nw if last else None, out_dtype=dt,
-                                            want_cast=L.side is not None)
-            if L.side is not None:
-                y = L.side(xc, ctx)
-                h, _ = M.add_rms_norm_rows(x, y, L.side.norm, eps, add_vec=nvec, next_w=nw,
-                                           out_dtype=dt)
-            if tap is not None:
-                tap.append(x.clone())
-        idx = meta.logits_indices
-        rows = x.index_select(0, idx) if idx.numel() != x.shape[0] else x
-        if rows.shape[0] == 0:
-            return rows.to(dt)
-        return M.rms_norm_rows(rows, self.final_norm, eps, dt)
-
-    def compute_logits(self, h: torch.Tensor) -> torch.Tensor:
-        """fp32 logits [rows, vocab rounded up to a multiple of 8]; columns past the
-        vocabulary are -inf."""
-        logits = self._head_product(h)
-        if self.vocab_pad:
-            logits[:, self.cfg.vocab_size:] = float("-inf")
-        return logits
-
-    def _head_product(self, h: torch.Tensor) -> torch.Tensor:
-        if h.dtype == torch.float32:
-            return F.linear(h, self.head)
-        # bf16 operands, fp32 accumulation and fp32 output
-        if h.is_cuda and self._mm_out_dtype:
-            try:
-                return torch.mm(h, self.head.t(), out_dtype=torch.float32)
-            except (TypeError, RuntimeError):
-                self._mm_out_dtype = False   # this build has no fp32-output bf16 product
-        return F.linear(h.float(), self.head.float())
+    def random_tensors(self, seed: int, device):
+        return random_tensors(self.cfg, seed, torch.bfloat16, device=device)
 
 
 # ---------------------------------------------------------------------------------------

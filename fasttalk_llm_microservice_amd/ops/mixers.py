@@ -1,6 +1,8 @@
 """Sequence-mixer and mixture-of-experts ops: latent (low-rank KV) attention over a
-paged latent cache, the gated delta-rule recurrence with per-channel decay over state
-slots, short causal convolutions, grouped top-k routing, clamped-GLU experts, and the
+paged latent cache, windowed attention (softmax or sigmoid weights, distance bias,
+several score maps per head) over a paged key / value cache, the gated delta-rule
+recurrence with per-channel decay and the selective state-space scan over state slots,
+short causal convolutions, grouped top-k routing, clamped-GLU experts, and the
 fp32-residual norms that tie them together.
 
 GPU tensors run the gfx950 kernels of the ``_C_mixers`` extension (``csrc/mixers``),
@@ -69,13 +71,13 @@ class Segments:
 # residual stream (fp32) and norms
 # ---------------------------------------------------------------------------------
 
-def embed_rows(ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
-    """fp32 residual rows table[ids]."""
+def embed_rows(ids: torch.Tensor, table: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
+    """fp32 residual rows table[ids] * scale."""
     if ids.is_cuda:
         out = torch.empty(ids.shape[0], table.shape[1], dtype=torch.float32, device=ids.device)
-        native_mixers().embed_rows(out, ids, table)
+        native_mixers().embed_rows(out, ids, table, float(scale))
         return out
-    return ref.embed_rows(ids, table)
+    return ref.embed_rows(ids, table, scale)
 
 
 def rms_norm_rows(x: torch.Tensor, w: torch.Tensor, eps: float, out_dtype,
@@ -114,16 +116,18 @@ rope_table = ref.rope_table
 # short convolution + gated delta rule (recurrent state slots)
 # ---------------------------------------------------------------------------------
 
-def short_conv_silu(x: torch.Tensor, conv_w: torch.Tensor, conv_state: torch.Tensor, seg: Segments):
-    """Per-channel causal convolution over time, then SiLU.  ``conv_w`` [C, taps] fp32
-    (last column = the current row); ``conv_state`` [slots, taps-1, C] fp32 holds each
-    sequence's last inputs and is updated; a segment at position 0 starts from zeros."""
+def short_conv_silu(x: torch.Tensor, conv_w: torch.Tensor, conv_state: torch.Tensor, seg: Segments,
+                    bias: Optional[torch.Tensor] = None):
+    """Per-channel causal convolution over time (+ ``bias`` [C] fp32), then SiLU.
+    ``conv_w`` [C, taps] fp32 (last column = the current row); ``conv_state`` [slots,
+    taps-1, C] fp32 holds each sequence's last inputs and is updated; a segment at
+    position 0 starts from zeros.  ``x`` may be a column range of wider rows."""
     if x.is_cuda:
-        out = torch.empty_like(x)
-        native_mixers().short_conv_silu(out, x, conv_w, conv_state, seg.start, seg.pos0, seg.slot,
+        out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+        native_mixers().short_conv_silu(out, x, conv_w, bias, conv_state, seg.start, seg.pos0, seg.slot,
                                         seg.num, seg.max_rows)
         return out
-    return ref.short_conv_silu(x, conv_w, conv_state, seg)
+    return ref.short_conv_silu(x, conv_w, conv_state, seg, bias)
 
 
 def gated_delta_rule(qkv, a, b, a_log, dt_bias, state, seg: Segments, heads: int, kv_heads: int,
@@ -263,6 +267,177 @@ def latent_attention_products(out, qa, qr, cache, seg: Segments, scale: float, r
 
 
 # ---------------------------------------------------------------------------------
+# selective state-space scan (recurrent state slots)
+# ---------------------------------------------------------------------------------
+
+def ssd_scan(xbc, dt, a_log, dt_bias, d_skip, state, seg: Segments, heads: int, groups: int, n: int,
+             dv: int) -> torch.Tensor:
+    """State-space recurrence with one scalar decay per head and row.
+
+    Rows of ``xbc`` are [x (heads*dv) | B (groups*n) | C (groups*n)] after the short
+    convolution; ``dt`` [T, heads] is the raw step projection (may be a column range).
+    step = softplus(dt + dt_bias), decay = exp(-exp(a_log) * step); per head (group
+    floor(h / (heads / groups))) and row:  S <- decay S + step B x^T (S is n x dv);
+    y = S^T C + d_skip x.  ``state`` [slots, heads, n, dv] fp32 is read (zeros at
+    position 0) and left at the segment's last row.  Returns y fp32 [T, heads*dv]."""
+    if xbc.is_cuda:
+        y = torch.empty(xbc.shape[0], heads * dv, dtype=torch.float32, device=xbc.device)
+        native_mixers().ssd_scan(y, xbc, dt, a_log, dt_bias, d_skip, state, seg.start, seg.pos0, seg.slot,
+                                 seg.num, heads, groups, n, dv)
+        return y
+    return ref.ssd_scan(xbc, dt, a_log, dt_bias, d_skip, state, seg, heads, groups, n, dv)
+
+
+def gate_group_norm(y, z, w, eps: float, groups: int, out_dtype):
+    """v = y * silu(z); each of ``groups`` equal parts of a row divided by its own root
+    mean square; times w.  y fp32 [T, n], z [T, n] (may be a column range)."""
+    if y.is_cuda:
+        out = torch.empty(y.shape, dtype=out_dtype, device=y.device)
+        native_mixers().gate_group_norm(out, y, z, w, eps, groups)
+        return out
+    return ref.gate_group_norm(y, z, w, eps, groups, out_dtype)
+
+
+# ---------------------------------------------------------------------------------
+# windowed attention (paged key cache + paged value cache)
+# ---------------------------------------------------------------------------------
+
+def attn_prep(qkv, nq: int, nk: int, q_norm_w, k_norm_w, eps: float, table, rot_dims: int,
+              head_dim: int, positions, slot_mapping, k_cache, v_cache) -> torch.Tensor:
+    """Rows [q (nq) | k (nk) | v] of a fused projection -> fp32 queries [T, nq]; keys and
+    values go to the rows' cache slots.  Optional steps, in this order: RMS norm of the
+    whole q part and of the whole k part with weights ``q_norm_w`` / ``k_norm_w``; rotary
+    positions on the first ``rot_dims`` entries of every ``head_dim`` chunk of q and k
+    (entry i paired with i + rot_dims/2, ``table`` = :func:`rope_table`)."""
+    if qkv.is_cuda:
+        q = torch.empty(qkv.shape[0], nq, dtype=torch.float32, device=qkv.device)
+        native_mixers().attn_prep(q, qkv, nq, nk, q_norm_w, k_norm_w, eps, table, rot_dims, head_dim,
+                                  positions, slot_mapping, k_cache, v_cache)
+        return q
+    return ref.attn_prep(qkv, nq, nk, q_norm_w, k_norm_w, eps, table, rot_dims, head_dim, positions,
+                         slot_mapping, k_cache, v_cache)
+
+
+@dataclasses.dataclass
+class WindowSpec:
+    """A windowed attention's constants.  Query head a = h * maps + m (head h, score map
+    m) reads key head floor(h / (heads / kv_heads)) * maps + m and value head
+    floor(h / (heads / kv_heads)).  Position i sees j iff 0 <= i - j < window (window 0:
+    every earlier key).  score = q.k * scale - r1[a] ln(1 + r2[a] (i - j)); weight =
+    softmax over the visible keys, or sigmoid(score + pb[a]) without normalisation."""
+    heads: int
+    kv_heads: int
+    dk: int
+    dv: int
+    window: int
+    scale: float
+    maps: int = 1
+    sigmoid: bool = False
+    r1: Optional[torch.Tensor] = None     # fp32 [heads * maps] (with r2)
+    r2: Optional[torch.Tensor] = None
+    pb: Optional[torch.Tensor] = None     # fp32 [heads * maps] (sigmoid weights only)
+
+
+def window_attention(q, k_cache, v_cache, seg: Segments, spec: WindowSpec, skip_from: int = 0,
+                     out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """q fp32 [T, heads*maps*dk] against the paged caches; fp32 [T, heads*maps, dv].
+    ``skip_from`` > 0: segments of that many rows or more are left to the caller
+    (:func:`window_attention_products`)."""
+    sp = spec
+    if q.is_cuda:
+        if out is None:
+            out = torch.empty(q.shape[0], sp.heads * sp.maps, sp.dv, dtype=torch.float32, device=q.device)
+        native_mixers().window_attention(out, q, k_cache, v_cache, seg.start, seg.pos0, seg.kv_len,
+                                         seg.block_tables, seg.num, seg.max_rows, sp.heads, sp.maps,
+                                         sp.kv_heads, sp.dk, sp.dv, sp.window, sp.scale, sp.sigmoid,
+                                         sp.r1, sp.r2, sp.pb, skip_from)
+        return out
+    r = ref.window_attention(q, k_cache, v_cache, seg, sp.heads, sp.maps, sp.kv_heads, sp.dk, sp.dv,
+                             sp.window, sp.scale, sp.sigmoid, sp.r1, sp.r2, sp.pb)
+    if out is not None:
+        out.copy_(r)
+        return out
+    return r
+
+
+def band_weights(s, first_pos: int, key0: int, spec: WindowSpec, rep_rows: int):
+    """Raw dot products fp32 [kv_heads*maps, rep*rows, keys] (the query heads that share
+    a key head stacked along the rows, ``rep_rows`` = rows of one of them) -> attention
+    weights fp32, in place: row r of a head is position first_pos + r, column c is
+    position key0 + c."""
+    sp = spec
+    if s.is_cuda:
+        native_mixers().band_weights(s, rep_rows, first_pos, key0, sp.heads, sp.maps, sp.kv_heads,
+                                     sp.window, sp.scale, sp.sigmoid, sp.r1, sp.r2, sp.pb)
+        return s
+    g, rr, keys = s.shape
+    rep = sp.heads // sp.kv_heads
+    # [G, maps, rep, rows, keys] -> query-head order (g, r, m)
+    v = s.view(sp.kv_heads, sp.maps, rep, rep_rows, keys).permute(0, 2, 1, 3, 4) \
+        .reshape(sp.heads * sp.maps, rep_rows, keys)
+    w = ref.band_weights(v, first_pos, key0, sp.window, sp.scale, sp.sigmoid, sp.r1, sp.r2, sp.pb)
+    s.copy_(w.view(sp.kv_heads, rep, sp.maps, rep_rows, keys).permute(0, 2, 1, 3, 4).reshape(g, rr, keys))
+    return s
+
+
+def window_attention_products(out, q, k_cache, v_cache, seg: Segments, spec: WindowSpec, min_rows: int):
+    """Segments of ``min_rows`` rows or more as banded matrix products: a chunk of rows
+    [c0, c1) only sees the keys c0 - window + 1 .. c1 - 1, so per chunk and key head the
+    scores are one product with M = (query heads of the group) x rows, the weights come
+    from :func:`band_weights` (fp32) and the sums are a second product with the value
+    head.  Operands are fp32 (cached rows are widened), so scores, weights and sums are
+    true fp32.  Needs the segments' host copies; writes its rows of ``out``."""
+    sp = spec
+    start, pos0, kv_len = seg.host
+    bs = k_cache.shape[1]
+    rep = sp.heads // sp.kv_heads
+    gk = sp.kv_heads * sp.maps
+    for s in range(seg.num):
+        a, b = start[s], start[s + 1]
+        n = b - a
+        if n < min_rows:
+            continue
+        step = PRODUCT_CHUNK_ROWS if sp.window <= 0 else max(PRODUCT_CHUNK_ROWS, min(sp.window, 1024))
+        for c0 in range(0, n, step):
+            c1 = min(n, c0 + step)
+            rows = c1 - c0
+            i0 = pos0[s] + c0
+            lo = max(0, i0 - sp.window + 1) if sp.window > 0 else 0
+            hi = min(kv_len[s], pos0[s] + c1)
+            b0, b1 = lo // bs, (hi + bs - 1) // bs
+            blocks = seg.block_tables[s, b0:b1].long()
+            off = lo - b0 * bs
+            k = k_cache.index_select(0, blocks).view((b1 - b0) * bs, gk, sp.dk)[off:off + hi - lo].float()
+            v = v_cache.index_select(0, blocks).view((b1 - b0) * bs, sp.kv_heads, sp.dv)[off:off + hi - lo].float()
+            # q rows [rows, (g, r, m), dk] -> [(g, m), (r, rows), dk]
+            qc = q[a + c0:a + c1].view(rows, sp.kv_heads, rep, sp.maps, sp.dk).permute(1, 3, 2, 0, 4) \
+                .reshape(gk, rep * rows, sp.dk)
+            sc = torch.bmm(qc, k.permute(1, 2, 0))                       # [gk, rep*rows, keys]
+            band_weights(sc, i0, lo, sp, rows)
+            # both maps of a group read the same value head: [G, maps*rep*rows, keys] x [G, keys, dv]
+            o = torch.bmm(sc.view(sp.kv_heads, sp.maps * rep * rows, hi - lo), v.transpose(0, 1))
+            out[a + c0:a + c1] = o.view(sp.kv_heads, sp.maps, rep, rows, sp.dv).permute(3, 0, 2, 1, 4) \
+                .reshape(rows, sp.heads * sp.maps, sp.dv)
+    return out
+
+
+# rows of a segment that one pair of banded products covers (at least; a window wider
+# than this takes a chunk of its own width, up to 1024 rows)
+PRODUCT_CHUNK_ROWS = 256
+
+
+def diff_combine(a, gate, lam: float, post_scale: float, eps: float, heads: int, dv: int, out_dtype):
+    """Two score maps per head -> one output: o = a[:, 2h] - lam * a[:, 2h+1], divided by
+    its root mean square over dv, times post_scale * sigmoid(gate[:, h]).  a fp32
+    [T, heads*2, dv]; gate [T, heads] (may be a column range); [T, heads*dv]."""
+    if a.is_cuda:
+        out = torch.empty(a.shape[0], heads * dv, dtype=out_dtype, device=a.device)
+        native_mixers().diff_combine(out, a, gate, float(lam), float(post_scale), eps, heads, dv)
+        return out
+    return ref.diff_combine(a, gate, lam, post_scale, eps, heads, dv, out_dtype)
+
+
+# ---------------------------------------------------------------------------------
 # mixture of experts
 # ---------------------------------------------------------------------------------
 
@@ -297,6 +472,15 @@ def clamp_swiglu(gu, limit: float):
         native_mixers().clamp_swiglu(out, gu, float(limit))
         return out
     return ref.clamp_swiglu(gu, limit)
+
+
+def gelu_glu(gu):
+    """[gate | up] rows -> gelu_tanh(gate) * up."""
+    if gu.is_cuda:
+        out = torch.empty(gu.shape[0], gu.shape[1] // 2, dtype=gu.dtype, device=gu.device)
+        native_mixers().gelu_glu(out, gu)
+        return out
+    return ref.gelu_glu(gu)
 
 
 def relu_sq(x):

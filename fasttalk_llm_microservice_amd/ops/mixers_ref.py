@@ -14,8 +14,9 @@ import torch
 import torch.nn.functional as F
 
 
-def embed_rows(ids, table):
-    return table.index_select(0, ids.long()).float()
+def embed_rows(ids, table, scale=1.0):
+    x = table.index_select(0, ids.long()).float()
+    return x * scale if scale != 1.0 else x
 
 
 def _rms(x, eps):
@@ -37,11 +38,24 @@ def add_rms_norm_rows(residual, y, wb, eps, add_vec, next_w, out_dtype, want_cas
     return out, cast
 
 
-def rope_table(max_pos: int, dims: int, base: float, device=None):
+def scale_frequencies(f, factor: float, low: float, high: float, original: float):
+    """Long-context rescaling of rotary frequencies by wavelength l = 2 pi / f: kept
+    where l < original / high, divided by ``factor`` where l > original / low, and
+    blended linearly in ``original / l`` between the two."""
+    wl = 2.0 * math.pi / f
+    s = ((original / wl - low) / (high - low)).clamp(0.0, 1.0)
+    mid = (1.0 - s) * f / factor + s * f
+    return torch.where(wl < original / high, f, torch.where(wl > original / low, f / factor, mid))
+
+
+def rope_table(max_pos: int, dims: int, base: float, device=None, scaling=None):
     """fp32 [max_pos, dims] = [cos | sin]; frequencies, angles and their cos / sin are
-    all evaluated in fp32 (angle = float(p) * f_i, f_i = base^(-2i/dims))."""
+    all evaluated in fp32 (angle = float(p) * f_i, f_i = base^(-2i/dims));
+    ``scaling``: (factor, low, high, original) for :func:`scale_frequencies`."""
     i = torch.arange(dims // 2, dtype=torch.float32)
     f = torch.tensor(float(base), dtype=torch.float32) ** (-2.0 * i / dims)
+    if scaling is not None:
+        f = scale_frequencies(f, *[float(v) for v in scaling])
     a = torch.arange(max_pos, dtype=torch.float32)[:, None] * f[None]
     return torch.cat([a.cos(), a.sin()], -1).to(device)
 
@@ -54,10 +68,10 @@ def _rope(x, cs, dims):
     return torch.cat([u * cos - v * sin, v * cos + u * sin, x[..., dims:]], -1)
 
 
-def short_conv_silu(x, conv_w, conv_state, seg):
+def short_conv_silu(x, conv_w, conv_state, seg, bias=None):
     t, c = x.shape
     taps = conv_w.shape[1]
-    out = torch.empty_like(x)
+    out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
     w = conv_w.float()
     start = seg.start.tolist()
     for s in range(seg.num):
@@ -70,6 +84,8 @@ def short_conv_silu(x, conv_w, conv_state, seg):
         xp = torch.cat([hist, x[a:b].float()], 0)            # [taps-1 + n, C]
         n = b - a
         y = sum(xp[j:j + n] * w[:, j][None] for j in range(taps))
+        if bias is not None:
+            y = y + bias.float()
         out[a:b] = (y * torch.sigmoid(y)).to(x.dtype)
         if taps > 1:
             conv_state[slot] = xp[n:]
@@ -221,3 +237,125 @@ def scale_add_rows(out, y, rows, weights, sigmoid: bool):
         out.add_(upd)
     else:
         out.index_add_(0, rows.long(), upd)
+
+
+# ---------------------------------------------------------------------------------
+# windowed attention over a paged key / value cache, selective state space scan
+# ---------------------------------------------------------------------------------
+
+def attn_prep(qkv, nq, nk, q_norm_w, k_norm_w, eps, table, rot_dims, head_dim, positions, slot_mapping,
+              k_cache, v_cache):
+    t = qkv.shape[0]
+    x = qkv.float()
+    q, k, v = x[:, :nq], x[:, nq:nq + nk], x[:, nq + nk:]
+    if q_norm_w is not None:
+        q = _rms(q, eps) * q_norm_w.float()
+    if k_norm_w is not None:
+        k = _rms(k, eps) * k_norm_w.float()
+    if table is not None and rot_dims > 0:
+        cs = table[positions[:t].long()]
+        q = _rope(q.reshape(t, -1, head_dim).transpose(0, 1), cs, rot_dims).transpose(0, 1).reshape(t, nq)
+        k = _rope(k.reshape(t, -1, head_dim).transpose(0, 1), cs, rot_dims).transpose(0, 1).reshape(t, nk)
+    slots = slot_mapping[:t].long()
+    keep = slots >= 0
+    if keep.any():
+        k_cache.view(-1, k_cache.shape[-1])[slots[keep]] = k[keep].to(k_cache.dtype)
+        v_cache.view(-1, v_cache.shape[-1])[slots[keep]] = v[keep].to(v_cache.dtype)
+    return q.contiguous()
+
+
+def band_weights(s, first_pos, key0, window, scale, sigmoid, r1, r2, pb):
+    """s fp32 [heads, rows, keys] raw dot products -> attention weights: row r is position
+    first_pos + r, column c is position key0 + c, visible iff 0 <= i - j (< window)."""
+    heads, rows, keys = s.shape
+    dist = (first_pos + torch.arange(rows, device=s.device))[:, None] - \
+        (key0 + torch.arange(keys, device=s.device))[None, :]
+    vis = dist >= 0
+    if window > 0:
+        vis &= dist < window
+    z = s * scale
+    if r1 is not None:
+        z = z - r1.float()[:, None, None] * torch.log(1.0 + r2.float()[:, None, None]
+                                                      * dist.clamp_min(0).float()[None])
+    if sigmoid:
+        if pb is not None:
+            z = z + pb.float()[:, None, None]
+        return torch.sigmoid(z) * vis[None]
+    z = z.masked_fill(~vis[None], float("-inf"))
+    return torch.softmax(z, -1).masked_fill(~vis[None], 0.0)
+
+
+def window_attention(q, k_cache, v_cache, seg, heads, maps, kv_heads, dk, dv, window, scale, sigmoid,
+                     r1, r2, pb):
+    """q fp32 [T, heads*maps*dk]; caches [blocks, bs, kv_heads*maps*dk] / [blocks, bs,
+    kv_heads*dv]; returns fp32 [T, heads*maps, dv]."""
+    t = q.shape[0]
+    hq = heads * maps
+    rep = heads // kv_heads
+    out = torch.zeros(t, hq, dv, dtype=torch.float32, device=q.device)
+    bs = k_cache.shape[1]
+    start = seg.start.tolist()
+    a_idx = torch.arange(hq)
+    khead = (a_idx // maps // rep) * maps + a_idx % maps
+    vhead = a_idx // maps // rep
+    for s in range(seg.num):
+        a, b = start[s], start[s + 1]
+        n = int(seg.kv_len[s])
+        if b == a or n == 0:
+            continue
+        p0 = int(seg.pos0[s])
+        lo = max(0, p0 - window + 1) if window > 0 else 0
+        nblk = (n + bs - 1) // bs
+        blocks = seg.block_tables[s, :nblk].long()
+        k = k_cache[blocks].reshape(nblk * bs, -1)[lo:n].float().view(n - lo, kv_heads * maps, dk)
+        v = v_cache[blocks].reshape(nblk * bs, -1)[lo:n].float().view(n - lo, kv_heads, dv)
+        qs = q[a:b].view(b - a, hq, dk)
+        sc = torch.einsum("thd,jhd->htj", qs, k[:, khead])
+        w = band_weights(sc, p0, lo, window, scale, sigmoid, r1, r2, pb)
+        out[a:b] = torch.einsum("htj,jhd->thd", w, v[:, vhead])
+    return out
+
+
+def diff_combine(a, gate, lam, post_scale, eps, heads, dv, out_dtype):
+    t = a.shape[0]
+    x = a.view(t, heads, 2, dv)
+    o = x[:, :, 0] - lam * x[:, :, 1]
+    o = _rms(o, eps) * post_scale * torch.sigmoid(gate.float())[:, :, None]
+    return o.reshape(t, heads * dv).to(out_dtype)
+
+
+def ssd_scan(xbc, dt, a_log, dt_bias, d_skip, state, seg, heads, groups, n, dv):
+    t = xbc.shape[0]
+    inner = heads * dv
+    f = xbc.float()
+    x = f[:, :inner].view(t, heads, dv)
+    bm = f[:, inner:inner + groups * n].view(t, groups, n)
+    cm = f[:, inner + groups * n:].view(t, groups, n)
+    step = F.softplus(dt.float() + dt_bias.float(), threshold=1e9)
+    decay = torch.exp(-torch.exp(a_log.float())[None] * step)
+    grp = torch.arange(heads) // (heads // groups)
+    y = torch.zeros(t, heads, dv, dtype=torch.float32, device=xbc.device)
+    start = seg.start.tolist()
+    for s in range(seg.num):
+        slot = int(seg.slot[s])
+        if slot < 0:
+            continue
+        S = state[slot] if int(seg.pos0[s]) > 0 else torch.zeros_like(state[slot])
+        for r in range(start[s], start[s + 1]):
+            S = decay[r][:, None, None] * S + (step[r][:, None] * bm[r, grp])[:, :, None] * x[r][:, None, :]
+            y[r] = (S * cm[r, grp][:, :, None]).sum(1) + d_skip.float()[:, None] * x[r]
+        state[slot] = S
+    return y.view(t, inner)
+
+
+def gate_group_norm(y, z, w, eps, groups, out_dtype):
+    t, inner = y.shape
+    zf = z.float()
+    v = y * (zf * torch.sigmoid(zf))
+    v = _rms(v.view(t, groups, inner // groups), eps).view(t, inner) * w.float()
+    return v.to(out_dtype)
+
+
+def gelu_glu(gu):
+    ff = gu.shape[1] // 2
+    return (gelu_tanh(gu[:, :ff].float()) * gu[:, ff:].float()).to(gu.dtype)
