@@ -11,7 +11,30 @@
 
 extern "C" {
 int mx_embed_rows(float* out, const int* ids, const void* table, int bf16, int rows, int width, int vocab,
-                  hipStream_t s);
+                  float scale, hipStream_t s);
+int mx_gelu_glu(void* out, const void* gu, int bf16, long gu_stride, long rows, int ff, hipStream_t s);
+int mx_attn_prep(float* q_out, const void* qkv, int bf16, long stride, int nq, int nk, int nv, const float* wq,
+                 const float* wk, float eps, const float* table, int table_rows, int rot_dims, int head_dim,
+                 const int* positions, const int* slots, void* k_cache, void* v_cache, int cache_bf16,
+                 long num_slots, long rows, hipStream_t s);
+int mx_window_max_dv();
+int mx_window_attention(float* out, const float* q, const void* k_cache, const void* v_cache, int cache_bf16,
+                        const int* start, const int* pos0, const int* kv_len, const int* bt, int bt_stride,
+                        int num_segs, long total_rows, int heads, int maps, int kv_heads, int dk, int dv, int window,
+                        float scale, int sigmoid, const float* r1, const float* r2, const float* pb, int block_size,
+                        int num_blocks, int skip_from, hipStream_t s);
+int mx_band_weights(float* S, int gk, int rep_rows_total, int rows, int keys, int first_pos, int key0, int heads,
+                    int maps, int kv_heads, int window, float scale, int sigmoid, const float* r1, const float* r2,
+                    const float* pb, hipStream_t s);
+int mx_diff_combine(void* out, int out_bf16, const float* a, const void* gate, int gate_bf16, long gate_stride,
+                    long rows, int heads, int dv, float lam, float post, float eps, hipStream_t s);
+int mx_ssd_max_state();
+int mx_ssd_scan(float* y, const void* xbc, int bf16, long x_stride, const void* dt, long dt_stride,
+                const float* a_log, const float* dt_bias, const float* d_skip, float* state, const int* start,
+                const int* pos0, const int* slot, int num_segs, int heads, int groups, int n, int dv, int num_slots,
+                hipStream_t s);
+int mx_gate_group_norm(void* out, int out_bf16, const float* y, const void* z, int z_bf16, long z_stride,
+                       const float* w, long rows, int groups, int gs, float eps, hipStream_t s);
 int mx_add_rms_norm(float* x, const void* y, int y_bf16, long y_stride, const float* wb, const float* add_vec,
                     const float* next_w, void* out, void* cast, int out_bf16, int rows, int width, float eps,
                     hipStream_t s);
@@ -24,9 +47,9 @@ int mx_side_gate(void* out, const void* gpre, const void* table, int bf16, long 
                  int col0, long rows, int sd, int vocab, hipStream_t s);
 int mx_scale_add_rows(float* out, const void* y, int y_bf16, const int* rows, const void* weights, int w_bf16,
                       int sigmoid, long n, int width, int out_rows, hipStream_t s);
-int mx_short_conv_silu(void* out, const void* x, int bf16, const float* w, float* hist, const int* start,
-                       const int* pos0, const int* slot, int num_segs, int max_rows, int channels, int taps,
-                       int num_slots, hipStream_t s);
+int mx_short_conv_silu(void* out, const void* x, int bf16, long x_stride, const float* w, const float* bias,
+                       float* hist, const int* start, const int* pos0, const int* slot, int num_segs, int max_rows,
+                       int channels, int taps, int num_slots, hipStream_t s);
 int mx_delta_prep(float* qn, float* kn, float* g, float* beta, const void* qkv, int bf16, long qkv_stride,
                   const void* a, long a_stride, const void* b, long b_stride, const float* a_log,
                   const float* dt_bias, long rows, int heads, int kv_heads, int dk, hipStream_t s);
@@ -93,13 +116,13 @@ void check_segs(const Tensor& start, const Tensor& a, const Tensor& b, int64_t n
   TORCH_CHECK(num >= 0 && start.numel() >= num + 1 && a.numel() >= num && b.numel() >= num, "segment arrays too short");
 }
 
-void embed_rows(Tensor out, Tensor ids, Tensor table) {
+void embed_rows(Tensor out, Tensor ids, Tensor table, double scale) {
   check_f32(out, "out");
   check_i32(ids, "ids");
   TORCH_CHECK(table.is_cuda() && is_act(table) && table.is_contiguous() && table.dim() == 2, "table");
   TORCH_CHECK(out.dim() == 2 && out.size(0) == ids.numel() && out.size(1) == table.size(1), "out shape");
   chk(mx_embed_rows(out.data_ptr<float>(), ids.data_ptr<int>(), table.data_ptr(), bf(table), (int)ids.numel(),
-                    (int)table.size(1), (int)table.size(0), stream()), "embed_rows");
+                    (int)table.size(1), (int)table.size(0), (float)scale, stream()), "embed_rows");
 }
 
 void add_rms_norm(Tensor x, OptT y, OptT wb, OptT add_vec, OptT next_w, OptT out, OptT cast, double eps) {
@@ -191,19 +214,21 @@ void scale_add_rows(Tensor out, Tensor y, OptT rows, Tensor weights, bool sigmoi
                         (int)out.size(0), stream()), "scale_add_rows");
 }
 
-void short_conv_silu(Tensor out, Tensor x, Tensor w, Tensor hist, Tensor start, Tensor pos0, Tensor slot,
+void short_conv_silu(Tensor out, Tensor x, Tensor w, OptT bias, Tensor hist, Tensor start, Tensor pos0, Tensor slot,
                      int64_t num_segs, int64_t max_rows) {
-  TORCH_CHECK(x.is_cuda() && is_act(x) && x.is_contiguous() && x.dim() == 2, "x");
+  check_rows(x, "x");
   TORCH_CHECK(out.is_cuda() && out.is_contiguous() && out.scalar_type() == x.scalar_type() &&
               out.sizes() == x.sizes(), "out");
   check_f32(w, "conv_w");
+  if (bias) { check_f32(*bias, "conv bias"); TORCH_CHECK(bias->numel() == x.size(1), "conv bias size"); }
   check_f32(hist, "conv_state");
   const int64_t c = x.size(1), taps = w.size(1);
   TORCH_CHECK(w.dim() == 2 && w.size(0) == c && hist.dim() == 3 && hist.size(1) == taps - 1 && hist.size(2) == c,
               "conv shapes");
   check_segs(start, pos0, slot, num_segs);
   TORCH_CHECK(max_rows <= x.size(0), "max_rows");
-  chk(mx_short_conv_silu(out.data_ptr(), x.data_ptr(), bf(x), w.data_ptr<float>(), hist.data_ptr<float>(),
+  chk(mx_short_conv_silu(out.data_ptr(), x.data_ptr(), bf(x), x.stride(0), w.data_ptr<float>(),
+                         bias ? bias->data_ptr<float>() : nullptr, hist.data_ptr<float>(),
                          start.data_ptr<int>(), pos0.data_ptr<int>(), slot.data_ptr<int>(), (int)num_segs,
                          (int)max_rows, (int)c, (int)taps, (int)hist.size(0), stream()), "short_conv_silu");
 }
@@ -353,6 +378,142 @@ void moe_pairs(Tensor out, Tensor h, Tensor idx, Tensor wts, Tensor wgu, Tensor 
                    (int)width, (float)limit, stream()), "moe_pairs");
 }
 
+void gelu_glu(Tensor out, Tensor gu) {
+  check_rows(gu, "gu");
+  const int64_t ff = gu.size(1) / 2;
+  TORCH_CHECK(out.is_cuda() && out.is_contiguous() && out.scalar_type() == gu.scalar_type() && out.dim() == 2 &&
+              out.size(0) == gu.size(0) && out.size(1) == ff && ff >= 1 && gu.size(1) == 2 * ff, "out");
+  chk(mx_gelu_glu(out.data_ptr(), gu.data_ptr(), bf(gu), gu.stride(0), gu.size(0), (int)ff, stream()), "gelu_glu");
+}
+
+const float* opt_f32(const OptT& t, int64_t n, const char* what) {
+  if (!t) return nullptr;
+  check_f32(*t, what);
+  TORCH_CHECK(t->numel() == n, what, ": size");
+  return t->data_ptr<float>();
+}
+
+// paged caches [blocks, block_size, row]
+void check_cache(const Tensor& c, int64_t row, const char* n) {
+  TORCH_CHECK(c.is_cuda() && c.is_contiguous() && c.dim() == 3 && c.size(2) == row && is_act(c) &&
+              c.size(0) * c.size(1) < (1LL << 31), n, ": paged cache [blocks, block_size, ", row, "]");
+}
+
+void attn_prep(Tensor q, Tensor qkv, int64_t nq, int64_t nk, OptT wq, OptT wk, double eps, OptT table,
+               int64_t rot_dims, int64_t head_dim, Tensor positions, Tensor slots, Tensor k_cache, Tensor v_cache) {
+  check_f32(q, "q");
+  check_rows(qkv, "qkv");
+  check_i32(positions, "positions");
+  check_i32(slots, "slot_mapping");
+  const int64_t t = qkv.size(0), nv = qkv.size(1) - nq - nk;
+  TORCH_CHECK(nq >= 1 && nk >= 1 && nv >= 1 && head_dim >= 1 && nq % head_dim == 0 && nk % head_dim == 0 &&
+              rot_dims >= 0 && rot_dims % 2 == 0 && rot_dims <= head_dim && q.numel() == t * nq &&
+              positions.numel() >= t && slots.numel() >= t, "attn_prep shapes");
+  check_cache(k_cache, nk, "k_cache");
+  check_cache(v_cache, nv, "v_cache");
+  TORCH_CHECK(k_cache.scalar_type() == v_cache.scalar_type() && k_cache.size(0) == v_cache.size(0) &&
+              k_cache.size(1) == v_cache.size(1), "k / v caches differ");
+  const float* tp = nullptr;
+  int64_t trows = 0;
+  if (table && rot_dims > 0) {
+    check_f32(*table, "rope table");
+    TORCH_CHECK(table->dim() == 2 && table->size(1) == rot_dims, "rope table shape");
+    tp = table->data_ptr<float>();
+    trows = table->size(0);
+  }
+  chk(mx_attn_prep(q.data_ptr<float>(), qkv.data_ptr(), bf(qkv), qkv.stride(0), (int)nq, (int)nk, (int)nv,
+                   opt_f32(wq, nq, "q norm"), opt_f32(wk, nk, "k norm"), (float)eps, tp, (int)trows, (int)rot_dims,
+                   (int)head_dim, positions.data_ptr<int>(), slots.data_ptr<int>(), k_cache.data_ptr(),
+                   v_cache.data_ptr(), bf(k_cache), k_cache.size(0) * k_cache.size(1), t, stream()), "attn_prep");
+}
+
+void window_attention(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache, Tensor start, Tensor pos0, Tensor kv_len,
+                      Tensor bt, int64_t num_segs, int64_t max_rows, int64_t heads, int64_t maps, int64_t kv_heads,
+                      int64_t dk, int64_t dv, int64_t window, double scale, bool sigmoid, OptT r1, OptT r2, OptT pb,
+                      int64_t skip_from) {
+  check_f32(out, "out");
+  check_f32(q, "q");
+  TORCH_CHECK(heads >= 1 && maps >= 1 && kv_heads >= 1 && heads % kv_heads == 0 && dk >= 1 && dv >= 1 &&
+              dv <= mx_window_max_dv(), "window attention sizes");
+  const int64_t hq = heads * maps, t = q.size(0);
+  TORCH_CHECK(q.dim() == 2 && q.size(1) == hq * dk && out.numel() == t * hq * dv, "q / out");
+  check_cache(k_cache, kv_heads * maps * dk, "k_cache");
+  check_cache(v_cache, kv_heads * dv, "v_cache");
+  TORCH_CHECK(k_cache.scalar_type() == v_cache.scalar_type() && k_cache.size(0) == v_cache.size(0) &&
+              k_cache.size(1) == v_cache.size(1), "k / v caches differ");
+  check_segs(start, pos0, kv_len, num_segs);
+  check_i32(bt, "block tables");
+  TORCH_CHECK(bt.dim() == 2 && bt.size(0) >= num_segs && max_rows <= t, "block tables / max_rows");
+  TORCH_CHECK((bool)r1 == (bool)r2, "r1 and r2 go together");
+  chk(mx_window_attention(out.data_ptr<float>(), q.data_ptr<float>(), k_cache.data_ptr(), v_cache.data_ptr(),
+                          bf(k_cache), start.data_ptr<int>(), pos0.data_ptr<int>(), kv_len.data_ptr<int>(),
+                          bt.data_ptr<int>(), (int)bt.size(1), (int)num_segs, t, (int)heads, (int)maps, (int)kv_heads,
+                          (int)dk, (int)dv, (int)window, (float)scale, sigmoid ? 1 : 0, opt_f32(r1, hq, "r1"),
+                          opt_f32(r2, hq, "r2"), opt_f32(pb, hq, "pb"), (int)k_cache.size(1), (int)k_cache.size(0),
+                          (int)skip_from, stream()), "window_attention");
+}
+
+void band_weights(Tensor S, int64_t rows, int64_t first_pos, int64_t key0, int64_t heads, int64_t maps,
+                  int64_t kv_heads, int64_t window, double scale, bool sigmoid, OptT r1, OptT r2, OptT pb) {
+  check_f32(S, "S");
+  TORCH_CHECK(S.dim() == 3 && heads >= 1 && kv_heads >= 1 && heads % kv_heads == 0 && maps >= 1 &&
+              S.size(0) == kv_heads * maps && rows >= 1 && S.size(1) == heads / kv_heads * rows && first_pos >= 0 &&
+              key0 >= 0, "band_weights shapes");
+  TORCH_CHECK((bool)r1 == (bool)r2, "r1 and r2 go together");
+  const int64_t hq = heads * maps;
+  chk(mx_band_weights(S.data_ptr<float>(), (int)S.size(0), (int)S.size(1), (int)rows, (int)S.size(2), (int)first_pos,
+                      (int)key0, (int)heads, (int)maps, (int)kv_heads, (int)window, (float)scale, sigmoid ? 1 : 0,
+                      opt_f32(r1, hq, "r1"), opt_f32(r2, hq, "r2"), opt_f32(pb, hq, "pb"), stream()), "band_weights");
+}
+
+void diff_combine(Tensor out, Tensor a, Tensor gate, double lam, double post, double eps, int64_t heads, int64_t dv) {
+  check_f32(a, "a");
+  check_rows(gate, "gate");
+  const int64_t t = gate.size(0);
+  TORCH_CHECK(a.numel() == t * heads * 2 * dv && gate.size(1) == heads, "diff_combine shapes");
+  TORCH_CHECK(out.is_cuda() && is_act(out) && out.is_contiguous() && out.numel() == t * heads * dv &&
+              bf(out) == bf(gate), "out");
+  chk(mx_diff_combine(out.data_ptr(), bf(out), a.data_ptr<float>(), gate.data_ptr(), bf(gate), gate.stride(0), t,
+                      (int)heads, (int)dv, (float)lam, (float)post, (float)eps, stream()), "diff_combine");
+}
+
+void ssd_scan(Tensor y, Tensor xbc, Tensor dt, Tensor a_log, Tensor dt_bias, Tensor d_skip, Tensor state,
+              Tensor start, Tensor pos0, Tensor slot, int64_t num_segs, int64_t heads, int64_t groups, int64_t n,
+              int64_t dv) {
+  check_f32(y, "y");
+  check_rows(xbc, "xbc");
+  check_rows(dt, "dt");
+  check_f32(a_log, "a_log");
+  check_f32(dt_bias, "dt_bias");
+  check_f32(d_skip, "D");
+  check_f32(state, "state");
+  const int64_t t = xbc.size(0);
+  TORCH_CHECK(heads >= 1 && groups >= 1 && heads % groups == 0 && n >= 1 && n <= mx_ssd_max_state() && dv >= 1,
+              "state-space sizes");
+  TORCH_CHECK(xbc.size(1) == heads * dv + 2 * groups * n && dt.size(0) == t && dt.size(1) == heads &&
+              dt.scalar_type() == xbc.scalar_type() && a_log.numel() == heads && dt_bias.numel() == heads &&
+              d_skip.numel() == heads && y.numel() == t * heads * dv, "state-space shapes");
+  TORCH_CHECK(state.dim() == 4 && state.size(1) == heads && state.size(2) == n && state.size(3) == dv, "state");
+  check_segs(start, pos0, slot, num_segs);
+  chk(mx_ssd_scan(y.data_ptr<float>(), xbc.data_ptr(), bf(xbc), xbc.stride(0), dt.data_ptr(), dt.stride(0),
+                  a_log.data_ptr<float>(), dt_bias.data_ptr<float>(), d_skip.data_ptr<float>(),
+                  state.data_ptr<float>(), start.data_ptr<int>(), pos0.data_ptr<int>(), slot.data_ptr<int>(),
+                  (int)num_segs, (int)heads, (int)groups, (int)n, (int)dv, (int)state.size(0), stream()), "ssd_scan");
+}
+
+void gate_group_norm(Tensor out, Tensor y, Tensor z, Tensor w, double eps, int64_t groups) {
+  check_f32(y, "y");
+  check_rows(z, "z");
+  check_f32(w, "w");
+  TORCH_CHECK(y.dim() == 2 && z.size(0) == y.size(0) && z.size(1) == y.size(1) && w.numel() == y.size(1) &&
+              groups >= 1 && y.size(1) % groups == 0, "gate_group_norm shapes");
+  TORCH_CHECK(out.is_cuda() && is_act(out) && out.is_contiguous() && out.sizes() == y.sizes() && bf(out) == bf(z),
+              "out");
+  chk(mx_gate_group_norm(out.data_ptr(), bf(out), y.data_ptr<float>(), z.data_ptr(), bf(z), z.stride(0),
+                         w.data_ptr<float>(), y.size(0), (int)groups, (int)(y.size(1) / groups), (float)eps, stream()),
+      "gate_group_norm");
+}
+
 }  // namespace
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
@@ -371,6 +532,15 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("causal_softmax", &causal_softmax);
   m.def("moe_topk", &moe_topk);
   m.def("moe_pairs", &moe_pairs);
+  m.def("gelu_glu", &gelu_glu);
+  m.def("attn_prep", &attn_prep);
+  m.def("window_attention", &window_attention);
+  m.def("band_weights", &band_weights);
+  m.def("diff_combine", &diff_combine);
+  m.def("ssd_scan", &ssd_scan);
+  m.def("gate_group_norm", &gate_group_norm);
+  m.def("window_max_dv", []() { return (int64_t)mx_window_max_dv(); });
+  m.def("ssd_max_state", []() { return (int64_t)mx_ssd_max_state(); });
   m.def("delta_max_dk", []() { return (int64_t)mx_delta_max_dk(); });
   m.def("latent_max_rank", []() { return (int64_t)mx_latent_max_rank(); });
 }

@@ -19,10 +19,12 @@ namespace mx {
 
 constexpr int kMaxTaps = 16;
 
-// out[row, c] = silu(sum_j w[c, j] * in(row - (taps-1) + j, c)), inputs before the
-// segment's first row come from the slot's history (zeros at position 0)
+// out[row, c] = silu(bias[c] + sum_j w[c, j] * in(row - (taps-1) + j, c)), inputs before
+// the segment's first row come from the slot's history (zeros at position 0); rows of x
+// are x_stride apart (a column range of a wider product), rows of out are dense
 template <typename T>
-__global__ void short_conv_kernel(T* __restrict__ out, const T* __restrict__ x, const float* __restrict__ w,
+__global__ void short_conv_kernel(T* __restrict__ out, const T* __restrict__ x, long x_stride,
+                                  const float* __restrict__ w, const float* __restrict__ bias,
                                   const float* __restrict__ hist, const int* __restrict__ start,
                                   const int* __restrict__ pos0, const int* __restrict__ slot, int channels,
                                   int taps, int num_slots) {
@@ -40,11 +42,11 @@ __global__ void short_conv_kernel(T* __restrict__ out, const T* __restrict__ x, 
   }
   const bool fresh = pos0[s] <= 0;
   const float* h = hist + (long)sl * (taps - 1) * channels;
-  float acc = 0.f;
+  float acc = bias != nullptr ? bias[c] : 0.f;
   for (int j = 0; j < taps; ++j) {
     const int src = rel - (taps - 1) + j;
     float v;
-    if (src >= 0) v = ld(x, (long)(r0 + src) * channels + c);
+    if (src >= 0) v = ld(x, (long)(r0 + src) * x_stride + c);
     else v = fresh ? 0.f : h[(long)(taps - 1 + src) * channels + c];
     acc += v * w[(long)c * taps + j];
   }
@@ -54,7 +56,7 @@ __global__ void short_conv_kernel(T* __restrict__ out, const T* __restrict__ x, 
 // history <- the segment's last taps-1 inputs (older ones shift out); runs after
 // short_conv_kernel, one thread per (segment, channel)
 template <typename T>
-__global__ void conv_hist_kernel(const T* __restrict__ x, float* __restrict__ hist,
+__global__ void conv_hist_kernel(const T* __restrict__ x, long x_stride, float* __restrict__ hist,
                                  const int* __restrict__ start, const int* __restrict__ pos0,
                                  const int* __restrict__ slot, int channels, int taps, int num_slots) {
   const int s = blockIdx.y;
@@ -68,7 +70,7 @@ __global__ void conv_hist_kernel(const T* __restrict__ x, float* __restrict__ hi
   float keep[kMaxTaps];
   for (int m = 0; m < taps - 1; ++m) {
     const int src = n - (taps - 1) + m;
-    if (src >= 0) keep[m] = ld(x, (long)(r0 + src) * channels + c);
+    if (src >= 0) keep[m] = ld(x, (long)(r0 + src) * x_stride + c);
     else keep[m] = fresh ? 0.f : h[(long)(taps - 1 + src) * channels + c];
   }
   for (int m = 0; m < taps - 1; ++m) h[(long)m * channels + c] = keep[m];
@@ -268,7 +270,8 @@ delta_rule_kernel(float* __restrict__ o, const float* __restrict__ qn, const flo
 
 using namespace mx;
 
-extern "C" int mx_short_conv_silu(void* out, const void* x, int bf16, const float* w, float* hist,
+extern "C" int mx_short_conv_silu(void* out, const void* x, int bf16, long x_stride, const float* w,
+                                  const float* bias, float* hist,
                                   const int* start, const int* pos0, const int* slot, int num_segs,
                                   int max_rows, int channels, int taps, int num_slots, hipStream_t s) {
   if (num_segs <= 0 || max_rows <= 0 || channels <= 0) return 0;
@@ -276,12 +279,12 @@ extern "C" int mx_short_conv_silu(void* out, const void* x, int bf16, const floa
   const dim3 block(256);
   const dim3 grid((channels + 255) / 256, max_rows, num_segs);
   if (grid.y > 65535 || grid.z > 65535) return -2;
-  MX_DISPATCH_T(bf16, hipLaunchKernelGGL((short_conv_kernel<T>), grid, block, 0, s, (T*)out, (const T*)x, w,
-                                         hist, start, pos0, slot, channels, taps, num_slots));
+  MX_DISPATCH_T(bf16, hipLaunchKernelGGL((short_conv_kernel<T>), grid, block, 0, s, (T*)out, (const T*)x, x_stride,
+                                         w, bias, hist, start, pos0, slot, channels, taps, num_slots));
   if (taps > 1)
     MX_DISPATCH_T(bf16, hipLaunchKernelGGL((conv_hist_kernel<T>), dim3((channels + 255) / 256, num_segs),
-                                           block, 0, s, (const T*)x, hist, start, pos0, slot, channels,
-                                           taps, num_slots));
+                                           block, 0, s, (const T*)x, x_stride, hist, start, pos0, slot,
+                                           channels, taps, num_slots));
   return (int)hipGetLastError();
 }
 

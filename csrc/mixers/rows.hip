@@ -1,6 +1,6 @@
 // Row-wise kernels around an fp32 residual stream: embedding rows, the fused
 // "post-norm add + next pre-norm" step, per-head gated output norm, activations
-// (relu^2, clamped GLU, gelu * token-side embedding) and the weighted row scatter-add
+// (relu^2, clamped GLU, gelu GLU, gelu * token-side embedding) and the weighted row scatter-add
 // that combines expert outputs.
 #include "mx_common.h"
 
@@ -8,12 +8,12 @@ namespace mx {
 
 template <typename T>
 __global__ void embed_rows_kernel(float* __restrict__ out, const int* __restrict__ ids,
-                                  const T* __restrict__ table, int width, int vocab) {
+                                  const T* __restrict__ table, int width, int vocab, float scale) {
   const int row = blockIdx.x;
   int id = ids[row];
   if (id < 0 || id >= vocab) id = 0;
   for (int i = threadIdx.x; i < width; i += blockDim.x)
-    out[(long)row * width + i] = ld(table, (long)id * width + i);
+    out[(long)row * width + i] = ld(table, (long)id * width + i) * scale;
 }
 
 // residual (fp32, in place): x += rms_norm(y) * wb (+ add_vec);
@@ -106,6 +106,17 @@ __device__ __forceinline__ float gelu_tanh_(float z) {
   return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
 }
 
+// rows [gate (ff) | up (ff)]: out = gelu_tanh(gate) * up
+template <typename T>
+__global__ void gelu_glu_kernel(T* __restrict__ out, const T* __restrict__ gu, long gu_stride, long rows, int ff) {
+  const long n = rows * ff;
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) {
+    const long r = i / ff;
+    const int c = (int)(i % ff);
+    st(out, i, gelu_tanh_(ld(gu, r * gu_stride + c)) * ld(gu, r * gu_stride + ff + c));
+  }
+}
+
 template <typename T>
 __global__ void side_gate_kernel(T* __restrict__ out, const T* __restrict__ gpre,
                                  const T* __restrict__ table, long table_stride,
@@ -139,10 +150,10 @@ __global__ void scale_add_rows_kernel(float* __restrict__ out, const TY* __restr
 using namespace mx;
 
 extern "C" int mx_embed_rows(float* out, const int* ids, const void* table, int bf16, int rows,
-                             int width, int vocab, hipStream_t s) {
+                             int width, int vocab, float scale, hipStream_t s) {
   if (rows <= 0) return 0;
   MX_DISPATCH_T(bf16, hipLaunchKernelGGL((embed_rows_kernel<T>), dim3(rows), dim3(256), 0, s, out, ids,
-                                         (const T*)table, width, vocab));
+                                         (const T*)table, width, vocab, scale));
   return (int)hipGetLastError();
 }
 
@@ -201,6 +212,13 @@ extern "C" int mx_clamp_swiglu(void* out, const void* gu, int bf16, long gu_stri
   if (rows * ff <= 0) return 0;
   MX_DISPATCH_T(bf16, hipLaunchKernelGGL((clamp_swiglu_kernel<T>), dim3(ew_grid(rows * ff)), dim3(256), 0,
                                          s, (T*)out, (const T*)gu, gu_stride, rows, ff, limit));
+  return (int)hipGetLastError();
+}
+
+extern "C" int mx_gelu_glu(void* out, const void* gu, int bf16, long gu_stride, long rows, int ff, hipStream_t s) {
+  if (rows * ff <= 0) return 0;
+  MX_DISPATCH_T(bf16, hipLaunchKernelGGL((gelu_glu_kernel<T>), dim3(ew_grid(rows * ff)), dim3(256), 0, s, (T*)out,
+                                         (const T*)gu, gu_stride, rows, ff));
   return (int)hipGetLastError();
 }
 

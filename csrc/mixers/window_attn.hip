@@ -1,0 +1,393 @@
+// Windowed grouped-query attention over a paged key cache and a paged value cache:
+// softmax or sigmoid weights, an optional logarithmic distance bias, and several score
+// maps per head that share the head's values (differential attention).
+//
+// Query head a = h * maps + m (head h, map m) reads key head (h / rep) * maps + m and
+// value head h / rep, rep = heads / kv_heads.  Position i sees key j iff 0 <= i - j
+// (< window when window > 0).  score = q.k * scale - r1[a] ln(1 + r2[a] (i - j));
+// weight = softmax over the visible keys, or sigmoid(score + pb[a]) unnormalised.
+// Queries, scores, weights and sums are fp32; the caches hold fp32 or bf16 rows.
+//
+// Kernels: attn_prep (whole-projection RMS norms, rotary positions, cache writes),
+// window_attn (one workgroup per (row, query head): decode rows and short segments),
+// band_weights (scores -> weights for the banded matrix products of long segments) and
+// diff_combine (two maps -> one gated, normed head output).
+#include "mx_common.h"
+
+namespace mx {
+
+// ---------------------------------------------------------------------------------
+// one workgroup per row of the fused [q | k | v] projection
+// ---------------------------------------------------------------------------------
+template <typename T, typename TC, int NT>
+__global__ void attn_prep_kernel(float* __restrict__ q_out, const T* __restrict__ qkv, long stride,
+                                 int nq, int nk, int nv, const float* __restrict__ wq,
+                                 const float* __restrict__ wk, float eps, const float* __restrict__ table,
+                                 int table_rows, int rot_dims, int head_dim,
+                                 const int* __restrict__ positions, const int* __restrict__ slots,
+                                 TC* __restrict__ k_cache, TC* __restrict__ v_cache, long num_slots) {
+  __shared__ float red[NT / 64];
+  const long row = blockIdx.x;
+  const T* in = qkv + row * stride;
+  float rq = 1.f, rk = 1.f;
+  if (wq != nullptr) {
+    float ss = 0.f;
+    for (int e = threadIdx.x; e < nq; e += NT) {
+      const float v = ld(in, e);
+      ss += v * v;
+    }
+    ss = block_sum<NT>(ss, red);
+    rq = 1.0f / sqrtf(ss / (float)nq + eps);
+  }
+  if (wk != nullptr) {
+    float ss = 0.f;
+    for (int e = threadIdx.x; e < nk; e += NT) {
+      const float v = ld(in, nq + e);
+      ss += v * v;
+    }
+    ss = block_sum<NT>(ss, red);
+    rk = 1.0f / sqrtf(ss / (float)nk + eps);
+  }
+  int pos = positions[row];
+  const bool rot = table != nullptr && rot_dims > 0;
+  if (pos < 0 || pos >= table_rows) pos = 0;
+  const float* cs = rot ? table + (long)pos * rot_dims : nullptr;
+  const int half = rot_dims / 2;
+  const long slot = slots[row];
+  const bool keep = slot >= 0 && slot < num_slots;
+  // q entries, then k entries
+  for (int e = threadIdx.x; e < nq + nk; e += NT) {
+    const bool is_q = e < nq;
+    const int off = is_q ? e : e - nq;
+    const float* w = is_q ? wq : wk;
+    const float r = is_q ? rq : rk;
+    const T* src = in + (is_q ? 0 : nq);
+    float v = ld(src, off) * (w != nullptr ? r * w[off] : 1.f);
+    if (rot) {
+      const int d = off % head_dim;
+      if (d < rot_dims) {
+        const int i = d < half ? d : d - half;
+        const int po = d < half ? off + half : off - half;
+        const float pv = ld(src, po) * (w != nullptr ? r * w[po] : 1.f);
+        const float c = cs[i], s = cs[half + i];
+        v = d < half ? v * c - pv * s : v * c + pv * s;
+      }
+    }
+    if (is_q) q_out[row * nq + off] = v;
+    else if (keep) st(k_cache, slot * nk + off, v);
+  }
+  if (keep)
+    for (int e = threadIdx.x; e < nv; e += NT) st(v_cache, slot * nv + e, ld(in, nq + nk + e));
+}
+
+// ---------------------------------------------------------------------------------
+// per-row attention: grid (rows, query heads), 256 threads = 4 waves.  A wave takes
+// every fourth chunk of 64 keys: lane = key for the scores (each lane walks its key's
+// cached row), lane = value column for the sums (rows read coalesced, the weight of
+// key jj broadcast from its lane), online softmax per wave, waves merged through LDS.
+// ---------------------------------------------------------------------------------
+constexpr int kWaves = 4;
+constexpr int kMaxVCols = 4;          // value columns per lane: dv <= 256
+
+template <typename TC>
+__device__ __forceinline__ float dot_row(const TC* __restrict__ kp, const float* __restrict__ q, int dk, bool vec);
+
+template <>
+__device__ __forceinline__ float dot_row<float>(const float* __restrict__ kp, const float* __restrict__ q, int dk,
+                                                bool vec) {
+  float acc = 0.f;
+  if (vec) {
+    for (int d = 0; d < dk; d += 4) {
+      const float4 k4 = *reinterpret_cast<const float4*>(kp + d);
+      acc += q[d] * k4.x + q[d + 1] * k4.y + q[d + 2] * k4.z + q[d + 3] * k4.w;
+    }
+  } else {
+    for (int d = 0; d < dk; ++d) acc += q[d] * kp[d];
+  }
+  return acc;
+}
+
+template <>
+__device__ __forceinline__ float dot_row<bf16_t>(const bf16_t* __restrict__ kp, const float* __restrict__ q, int dk,
+                                                 bool vec) {
+  float acc = 0.f;
+  if (vec) {
+    for (int d = 0; d < dk; d += 8) {
+      const uint4 u = *reinterpret_cast<const uint4*>(kp + d);
+      const uint32_t w[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+      for (int p = 0; p < 4; ++p) {
+        acc += q[d + 2 * p] * __uint_as_float(w[p] << 16);
+        acc += q[d + 2 * p + 1] * __uint_as_float(w[p] & 0xffff0000u);
+      }
+    }
+  } else {
+    for (int d = 0; d < dk; ++d) acc += q[d] * ld(kp, d);
+  }
+  return acc;
+}
+
+template <typename TC>
+__global__ void __launch_bounds__(64 * kWaves)
+window_attn_kernel(float* __restrict__ out, const float* __restrict__ q, const TC* __restrict__ k_cache,
+                   const TC* __restrict__ v_cache, const int* __restrict__ start, const int* __restrict__ pos0,
+                   const int* __restrict__ kv_len, const int* __restrict__ bt, int bt_stride, int num_segs,
+                   int heads, int maps, int kv_heads, int dk, int dv, int window, float scale, int sigmoid,
+                   const float* __restrict__ r1, const float* __restrict__ r2, const float* __restrict__ pb,
+                   int block_size, int num_blocks, int skip_from, int vec) {
+  extern __shared__ float smem[];
+  const int row = blockIdx.x, a = blockIdx.y;
+  const int hq = heads * maps;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  // the segment that owns this row: the last s with start[s] <= row
+  int lo_s = 0, hi_s = num_segs;
+  while (hi_s - lo_s > 1) {
+    const int mid = (lo_s + hi_s) >> 1;
+    if (start[mid] <= row) lo_s = mid; else hi_s = mid;
+  }
+  const int s = lo_s;
+  const int r0 = start[s], n = start[s + 1] - r0;
+  if (row >= start[num_segs] || (skip_from > 0 && n >= skip_from)) return;
+  float* q_s = smem;                         // [dk]
+  float* o_s = smem + dk;                    // [kWaves][dv]
+  float* ml_s = o_s + kWaves * dv;           // [kWaves][2]
+  const float* qp = q + ((long)row * hq + a) * dk;
+  for (int d = tid; d < dk; d += blockDim.x) q_s[d] = qp[d];
+  __syncthreads();
+  const int h = a / maps, m = a % maps, rep = heads / kv_heads;
+  const int kh = (h / rep) * maps + m, vh = h / rep;
+  const long nk = (long)kv_heads * maps * dk, nv = (long)kv_heads * dv;
+  const int i = pos0[s] + (row - r0);
+  const int last = min(i, kv_len[s] - 1);    // padding rows (empty context) see nothing
+  const int first = window > 0 ? max(0, i - window + 1) : 0;
+  const int nkeys = last - first + 1;
+  const float c1 = r1 != nullptr ? r1[a] : 0.f, c2 = r1 != nullptr ? r2[a] : 0.f;
+  const float bias = (sigmoid && pb != nullptr) ? pb[a] : 0.f;
+  const int* table = bt + (long)s * bt_stride;
+
+  float o[kMaxVCols];
+#pragma unroll
+  for (int u = 0; u < kMaxVCols; ++u) o[u] = 0.f;
+  float mx_ = -INFINITY, l_ = 0.f;
+  for (int c0 = wave * 64; c0 < nkeys; c0 += 64 * kWaves) {
+    const int cnt = min(64, nkeys - c0);
+    const int j = first + c0 + lane;
+    int slot = -1;
+    float z = -INFINITY;
+    if (lane < cnt) {
+      const int blk = table[j / block_size];
+      if (blk >= 0 && blk < num_blocks) {
+        slot = blk * block_size + j % block_size;
+        z = dot_row<TC>(k_cache + (long)slot * nk + (long)kh * dk, q_s, dk, vec != 0) * scale;
+        if (r1 != nullptr) z -= c1 * logf(1.0f + c2 * (float)(i - j));
+      }
+    }
+    float p;
+    if (sigmoid) {
+      p = slot >= 0 ? sigmoidf_(z + bias) : 0.f;
+    } else {
+      const float mn = fmaxf(mx_, ft::wave_max(z));
+      const float resc = mx_ == -INFINITY ? 0.f : expf(mx_ - mn);
+      p = (slot >= 0 && mn != -INFINITY) ? expf(z - mn) : 0.f;
+      l_ = l_ * resc + ft::wave_sum(p);
+#pragma unroll
+      for (int u = 0; u < kMaxVCols; ++u) o[u] *= resc;
+      mx_ = mn;
+    }
+    for (int jj = 0; jj < cnt; ++jj) {
+      const float pj = __shfl(p, jj);
+      const int sj = __shfl(slot, jj);
+      if (sj < 0) continue;
+      const TC* vp = v_cache + (long)sj * nv + (long)vh * dv;
+#pragma unroll
+      for (int u = 0; u < kMaxVCols; ++u) {
+        const int c = lane + 64 * u;
+        if (c < dv) o[u] += pj * ld(vp, c);
+      }
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < kMaxVCols; ++u) {
+    const int c = lane + 64 * u;
+    if (c < dv) o_s[wave * dv + c] = o[u];
+  }
+  if (lane == 0) {
+    ml_s[2 * wave] = mx_;
+    ml_s[2 * wave + 1] = l_;
+  }
+  __syncthreads();
+  float* op = out + ((long)row * hq + a) * dv;
+  for (int c = tid; c < dv; c += blockDim.x) {
+    float acc = 0.f;
+    if (sigmoid) {
+#pragma unroll
+      for (int w = 0; w < kWaves; ++w) acc += o_s[w * dv + c];
+    } else {
+      float mm = -INFINITY;
+#pragma unroll
+      for (int w = 0; w < kWaves; ++w) mm = fmaxf(mm, ml_s[2 * w]);
+      float l = 0.f;
+#pragma unroll
+      for (int w = 0; w < kWaves; ++w) {
+        const float f = ml_s[2 * w] == -INFINITY ? 0.f : expf(ml_s[2 * w] - mm);
+        l += ml_s[2 * w + 1] * f;
+        acc += o_s[w * dv + c] * f;
+      }
+      acc = l > 0.f ? acc / l : 0.f;
+    }
+    op[c] = acc;
+  }
+}
+
+// ---------------------------------------------------------------------------------
+// scores -> weights in place for the banded products.  S [gk = (g, m)] [(r, t)] [keys]:
+// the rep query heads of a key head stacked along the rows.  grid (rep * rows, gk).
+// ---------------------------------------------------------------------------------
+template <int NT>
+__global__ void band_weights_kernel(float* __restrict__ S, int rows, int keys, int first_pos, int key0,
+                                    int heads, int maps, int kv_heads, int window, float scale, int sigmoid,
+                                    const float* __restrict__ r1, const float* __restrict__ r2,
+                                    const float* __restrict__ pb) {
+  __shared__ float red[NT / 64];
+  const int rep = heads / kv_heads;
+  const int rr = blockIdx.x, gk = blockIdx.y;
+  const int r = rr / rows, t = rr % rows;
+  const int g = gk / maps, m = gk % maps;
+  const int a = (g * rep + r) * maps + m;
+  const int i = first_pos + t;
+  float* sp = S + ((long)gk * rep * rows + rr) * keys;
+  // visible columns [c_lo, c_hi]
+  const int c_hi = min(keys - 1, i - key0);
+  const int c_lo = window > 0 ? max(0, i - window + 1 - key0) : 0;
+  const float c1 = r1 != nullptr ? r1[a] : 0.f, c2 = r1 != nullptr ? r2[a] : 0.f;
+  auto score = [&](int c) {
+    float z = sp[c] * scale;
+    if (r1 != nullptr) z -= c1 * logf(1.0f + c2 * (float)(i - key0 - c));
+    return z;
+  };
+  for (int c = threadIdx.x; c < c_lo; c += NT) sp[c] = 0.f;
+  for (int c = c_hi + 1 + threadIdx.x; c < keys; c += NT) sp[c] = 0.f;
+  if (sigmoid) {
+    const float bias = pb != nullptr ? pb[a] : 0.f;
+    for (int c = c_lo + threadIdx.x; c <= c_hi; c += NT) sp[c] = sigmoidf_(score(c) + bias);
+    return;
+  }
+  float mx_ = -INFINITY;
+  for (int c = c_lo + threadIdx.x; c <= c_hi; c += NT) {
+    const float z = score(c);
+    sp[c] = z;                         // each thread re-reads only its own columns
+    mx_ = fmaxf(mx_, z);
+  }
+  mx_ = ft::wave_max(mx_);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = mx_;
+  __syncthreads();
+#pragma unroll
+  for (int w = 0; w < NT / 64; ++w) mx_ = fmaxf(mx_, red[w]);
+  float sum = 0.f;
+  for (int c = c_lo + threadIdx.x; c <= c_hi; c += NT) {
+    const float p = expf(sp[c] - mx_);
+    sp[c] = p;
+    sum += p;
+  }
+  sum = block_sum<NT>(sum, red);
+  const float inv = sum > 0.f ? 1.0f / sum : 0.f;
+  for (int c = c_lo + threadIdx.x; c <= c_hi; c += NT) sp[c] *= inv;
+}
+
+// one wave per (row, head): o = a1 - lam a2; o / rms(o) * post * sigmoid(gate)
+template <typename TG, typename TO>
+__global__ void diff_combine_kernel(TO* __restrict__ out, const float* __restrict__ a, const TG* __restrict__ gate,
+                                    long gate_stride, long pairs, int heads, int dv, float lam, float post,
+                                    float eps) {
+  const long pair = (long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (pair >= pairs) return;
+  const int lane = threadIdx.x & 63;
+  const long row = pair / heads;
+  const int h = (int)(pair % heads);
+  const float* a1 = a + ((row * heads + h) * 2) * dv;
+  const float* a2 = a1 + dv;
+  float ss = 0.f;
+  for (int c = lane; c < dv; c += 64) {
+    const float o = a1[c] - lam * a2[c];
+    ss += o * o;
+  }
+  ss = ft::wave_sum(ss);
+  const float f = 1.0f / sqrtf(ss / (float)dv + eps) * post * sigmoidf_(ld(gate, row * gate_stride + h));
+  for (int c = lane; c < dv; c += 64) st(out, (row * heads + h) * dv + c, (a1[c] - lam * a2[c]) * f);
+}
+
+}  // namespace mx
+
+using namespace mx;
+
+extern "C" int mx_attn_prep(float* q_out, const void* qkv, int bf16, long stride, int nq, int nk, int nv,
+                            const float* wq, const float* wk, float eps, const float* table, int table_rows,
+                            int rot_dims, int head_dim, const int* positions, const int* slots, void* k_cache,
+                            void* v_cache, int cache_bf16, long num_slots, long rows, hipStream_t s) {
+  if (rows <= 0) return 0;
+  if (head_dim < 1 || rot_dims < 0 || rot_dims > head_dim || rot_dims % 2 || nq % head_dim || nk % head_dim) return -1;
+  const dim3 grid((unsigned)rows), block(256);
+#define MX_PREP(T, TC)                                                                                     \
+  hipLaunchKernelGGL((attn_prep_kernel<T, TC, 256>), grid, block, 0, s, q_out, (const T*)qkv, stride, nq, nk, \
+                     nv, wq, wk, eps, table, table_rows, rot_dims, head_dim, positions, slots, (TC*)k_cache,  \
+                     (TC*)v_cache, num_slots)
+  if (bf16 && cache_bf16) MX_PREP(bf16_t, bf16_t);
+  else if (bf16) MX_PREP(bf16_t, float);
+  else if (cache_bf16) MX_PREP(float, bf16_t);
+  else MX_PREP(float, float);
+#undef MX_PREP
+  return (int)hipGetLastError();
+}
+
+extern "C" int mx_window_max_dv() { return 64 * kMaxVCols; }
+
+extern "C" int mx_window_attention(float* out, const float* q, const void* k_cache, const void* v_cache,
+                                   int cache_bf16, const int* start, const int* pos0, const int* kv_len,
+                                   const int* bt, int bt_stride, int num_segs, long total_rows, int heads, int maps,
+                                   int kv_heads, int dk, int dv, int window, float scale, int sigmoid,
+                                   const float* r1, const float* r2, const float* pb, int block_size,
+                                   int num_blocks, int skip_from, hipStream_t s) {
+  if (num_segs <= 0 || total_rows <= 0) return 0;
+  if (dv < 1 || dv > mx_window_max_dv() || dk < 1 || heads % kv_heads || maps < 1) return -1;
+  const int hq = heads * maps;
+  if (total_rows > 0x7fffffffL || hq > 65535) return -2;
+  const long es = cache_bf16 ? 2 : 4;
+  const long nk = (long)kv_heads * maps * dk;
+  const int vec = (dk * es) % 16 == 0 && (nk * es) % 16 == 0 && ((uintptr_t)k_cache) % 16 == 0;
+  const size_t shm = (size_t)(dk + kWaves * dv + 2 * kWaves) * sizeof(float);
+  if (shm > 64 * 1024) return -3;
+  const dim3 grid((unsigned)total_rows, (unsigned)hq), block(64 * kWaves);
+  MX_DISPATCH_T(cache_bf16, hipLaunchKernelGGL((window_attn_kernel<T>), grid, block, shm, s, out, q,
+                                               (const T*)k_cache, (const T*)v_cache, start, pos0, kv_len, bt,
+                                               bt_stride, num_segs, heads, maps, kv_heads, dk, dv, window, scale,
+                                               sigmoid, r1, r2, pb, block_size, num_blocks, skip_from, vec));
+  return (int)hipGetLastError();
+}
+
+extern "C" int mx_band_weights(float* S, int gk, int rep_rows_total, int rows, int keys, int first_pos, int key0,
+                               int heads, int maps, int kv_heads, int window, float scale, int sigmoid,
+                               const float* r1, const float* r2, const float* pb, hipStream_t s) {
+  if (gk <= 0 || rep_rows_total <= 0 || keys <= 0) return 0;
+  if (heads % kv_heads || gk != kv_heads * maps || rep_rows_total != heads / kv_heads * rows || gk > 65535) return -1;
+  hipLaunchKernelGGL((band_weights_kernel<256>), dim3((unsigned)rep_rows_total, (unsigned)gk), dim3(256), 0, s, S,
+                     rows, keys, first_pos, key0, heads, maps, kv_heads, window, scale, sigmoid, r1, r2, pb);
+  return (int)hipGetLastError();
+}
+
+extern "C" int mx_diff_combine(void* out, int out_bf16, const float* a, const void* gate, int gate_bf16,
+                               long gate_stride, long rows, int heads, int dv, float lam, float post, float eps,
+                               hipStream_t s) {
+  const long pairs = rows * heads;
+  if (pairs <= 0) return 0;
+  const dim3 grid((unsigned)((pairs + 3) / 4)), block(256);
+  if (gate_bf16 && out_bf16)
+    hipLaunchKernelGGL((diff_combine_kernel<bf16_t, bf16_t>), grid, block, 0, s, (bf16_t*)out, a,
+                       (const bf16_t*)gate, gate_stride, pairs, heads, dv, lam, post, eps);
+  else if (!gate_bf16 && !out_bf16)
+    hipLaunchKernelGGL((diff_combine_kernel<float, float>), grid, block, 0, s, (float*)out, a, (const float*)gate,
+                       gate_stride, pairs, heads, dv, lam, post, eps);
+  else
+    return -1;
+  return (int)hipGetLastError();
+}
