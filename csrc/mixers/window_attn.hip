@@ -83,11 +83,38 @@ __global__ void attn_prep_kernel(float* __restrict__ q_out, const T* __restrict_
 // ---------------------------------------------------------------------------------
 // per-row attention: grid (rows, query heads), 256 threads = 4 waves.  A wave takes
 // every fourth chunk of 64 keys: lane = key for the scores (each lane walks its key's
-// cached row), lane = value column for the sums (rows read coalesced, the weight of
-// key jj broadcast from its lane), online softmax per wave, waves merged through LDS.
+// cached row in 16-byte pieces), online softmax per wave, waves merged through LDS.
+// The weighted sums of the value rows come in two forms:
+//  * VEC (value rows are whole 16-byte pieces): a lane owns one 16-byte piece of the
+//    row (8 bf16 / 4 fp32 columns) of every (64 / LPK)-th key, LPK = pieces per row
+//    rounded up to a power of two; a pass loads 64 / LPK whole rows with one 16-byte
+//    load per lane, branch-free (a key past the chunk's end reads row 0 with weight 0),
+//    so several passes are in flight; the lanes that share a piece are summed at the end;
+//  * otherwise lane = value column, one key at a time.
 // ---------------------------------------------------------------------------------
 constexpr int kWaves = 4;
-constexpr int kMaxVCols = 4;          // value columns per lane: dv <= 256
+constexpr int kMaxVCols = 4;          // value columns per lane (scalar form): dv <= 256
+
+template <typename TC> struct Piece;
+template <> struct Piece<float> {
+  static constexpr int N = 4;
+  static __device__ __forceinline__ void load(const float* p, float* v) {
+    const float4 u = *reinterpret_cast<const float4*>(p);
+    v[0] = u.x; v[1] = u.y; v[2] = u.z; v[3] = u.w;
+  }
+};
+template <> struct Piece<bf16_t> {
+  static constexpr int N = 8;
+  static __device__ __forceinline__ void load(const bf16_t* p, float* v) {
+    const uint4 u = *reinterpret_cast<const uint4*>(p);
+    const uint32_t w[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      v[2 * i] = __uint_as_float(w[i] << 16);
+      v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+    }
+  }
+};
 
 template <typename TC>
 __device__ __forceinline__ float dot_row(const TC* __restrict__ kp, const float* __restrict__ q, int dk, bool vec);
@@ -127,14 +154,14 @@ __device__ __forceinline__ float dot_row<bf16_t>(const bf16_t* __restrict__ kp, 
   return acc;
 }
 
-template <typename TC>
+template <typename TC, bool VEC>
 __global__ void __launch_bounds__(64 * kWaves)
 window_attn_kernel(float* __restrict__ out, const float* __restrict__ q, const TC* __restrict__ k_cache,
                    const TC* __restrict__ v_cache, const int* __restrict__ start, const int* __restrict__ pos0,
                    const int* __restrict__ kv_len, const int* __restrict__ bt, int bt_stride, int num_segs,
                    int heads, int maps, int kv_heads, int dk, int dv, int window, float scale, int sigmoid,
                    const float* __restrict__ r1, const float* __restrict__ r2, const float* __restrict__ pb,
-                   int block_size, int num_blocks, int skip_from, int vec) {
+                   int block_size, int num_blocks, int skip_from, int vec, int lpk) {
   extern __shared__ float smem[];
   const int row = blockIdx.x, a = blockIdx.y;
   const int hq = heads * maps;
@@ -165,9 +192,14 @@ window_attn_kernel(float* __restrict__ out, const float* __restrict__ q, const T
   const float bias = (sigmoid && pb != nullptr) ? pb[a] : 0.f;
   const int* table = bt + (long)s * bt_stride;
 
-  float o[kMaxVCols];
+  constexpr int NO = VEC ? Piece<TC>::N : kMaxVCols;
+  float o[NO];
 #pragma unroll
-  for (int u = 0; u < kMaxVCols; ++u) o[u] = 0.f;
+  for (int u = 0; u < NO; ++u) o[u] = 0.f;
+  // VEC: this lane's piece of the value row and which key of a pass it reads
+  const int pieces = dv / Piece<TC>::N;
+  const int sg = lane & (lpk - 1), sub = lane / lpk, kpp = 64 / lpk;
+  const bool has_piece = sg < pieces;
   float mx_ = -INFINITY, l_ = 0.f;
   for (int c0 = wave * 64; c0 < nkeys; c0 += 64 * kWaves) {
     const int cnt = min(64, nkeys - c0);
@@ -191,25 +223,54 @@ window_attn_kernel(float* __restrict__ out, const float* __restrict__ q, const T
       p = (slot >= 0 && mn != -INFINITY) ? expf(z - mn) : 0.f;
       l_ = l_ * resc + ft::wave_sum(p);
 #pragma unroll
-      for (int u = 0; u < kMaxVCols; ++u) o[u] *= resc;
+      for (int u = 0; u < NO; ++u) o[u] *= resc;
       mx_ = mn;
     }
-    for (int jj = 0; jj < cnt; ++jj) {
-      const float pj = __shfl(p, jj);
-      const int sj = __shfl(slot, jj);
-      if (sj < 0) continue;
-      const TC* vp = v_cache + (long)sj * nv + (long)vh * dv;
+    if constexpr (VEC) {
+      const int passes = (cnt + kpp - 1) / kpp;
+#pragma unroll 4
+      for (int ps = 0; ps < passes; ++ps) {
+        const int jj = ps * kpp + sub;                  // < 64: a lane past cnt has weight 0, slot -1
+        const float pj = __shfl(p, jj);
+        const int sj = __shfl(slot, jj);
+        const bool ok = sj >= 0 && has_piece;
+        const TC* vp = v_cache + (ok ? (long)sj * nv + (long)vh * dv + sg * Piece<TC>::N : 0L);
+        float v[Piece<TC>::N];
+        Piece<TC>::load(vp, v);
+        const float w = ok ? pj : 0.f;
 #pragma unroll
-      for (int u = 0; u < kMaxVCols; ++u) {
-        const int c = lane + 64 * u;
-        if (c < dv) o[u] += pj * ld(vp, c);
+        for (int u = 0; u < Piece<TC>::N; ++u) o[u] += w * v[u];
+      }
+    } else {
+      for (int jj = 0; jj < cnt; ++jj) {
+        const float pj = __shfl(p, jj);
+        const int sj = __shfl(slot, jj);
+        if (sj < 0) continue;
+        const TC* vp = v_cache + (long)sj * nv + (long)vh * dv;
+#pragma unroll
+        for (int u = 0; u < kMaxVCols; ++u) {
+          const int c = lane + 64 * u;
+          if (c < dv) o[u] += pj * ld(vp, c);
+        }
       }
     }
   }
+  if constexpr (VEC) {
+    // lanes sub = 0, 1, ... hold partial sums of the same piece
+    for (int off = lpk; off < 64; off <<= 1) {
 #pragma unroll
-  for (int u = 0; u < kMaxVCols; ++u) {
-    const int c = lane + 64 * u;
-    if (c < dv) o_s[wave * dv + c] = o[u];
+      for (int u = 0; u < NO; ++u) o[u] += __shfl_xor(o[u], off);
+    }
+    if (sub == 0 && has_piece) {
+#pragma unroll
+      for (int u = 0; u < NO; ++u) o_s[wave * dv + sg * Piece<TC>::N + u] = o[u];
+    }
+  } else {
+#pragma unroll
+    for (int u = 0; u < kMaxVCols; ++u) {
+      const int c = lane + 64 * u;
+      if (c < dv) o_s[wave * dv + c] = o[u];
+    }
   }
   if (lane == 0) {
     ml_s[2 * wave] = mx_;
@@ -355,13 +416,23 @@ extern "C" int mx_window_attention(float* out, const float* q, const void* k_cac
   const long es = cache_bf16 ? 2 : 4;
   const long nk = (long)kv_heads * maps * dk;
   const int vec = (dk * es) % 16 == 0 && (nk * es) % 16 == 0 && ((uintptr_t)k_cache) % 16 == 0;
+  // value rows in whole 16-byte pieces, at most 64 per row: the vector form of the sums
+  const long nv = (long)kv_heads * dv;
+  const long pieces = dv * es / 16;
+  const bool vecv = (dv * es) % 16 == 0 && (nv * es) % 16 == 0 && ((uintptr_t)v_cache) % 16 == 0 && pieces <= 64;
+  int lpk = 1;
+  while (lpk < pieces) lpk <<= 1;
   const size_t shm = (size_t)(dk + kWaves * dv + 2 * kWaves) * sizeof(float);
   if (shm > 64 * 1024) return -3;
   const dim3 grid((unsigned)total_rows, (unsigned)hq), block(64 * kWaves);
-  MX_DISPATCH_T(cache_bf16, hipLaunchKernelGGL((window_attn_kernel<T>), grid, block, shm, s, out, q,
-                                               (const T*)k_cache, (const T*)v_cache, start, pos0, kv_len, bt,
-                                               bt_stride, num_segs, heads, maps, kv_heads, dk, dv, window, scale,
-                                               sigmoid, r1, r2, pb, block_size, num_blocks, skip_from, vec));
+#define MX_WATTN(V)                                                                                          \
+  MX_DISPATCH_T(cache_bf16, hipLaunchKernelGGL((window_attn_kernel<T, V>), grid, block, shm, s, out, q,         \
+                                               (const T*)k_cache, (const T*)v_cache, start, pos0, kv_len, bt,  \
+                                               bt_stride, num_segs, heads, maps, kv_heads, dk, dv, window, scale, \
+                                               sigmoid, r1, r2, pb, block_size, num_blocks, skip_from, vec, lpk))
+  if (vecv) MX_WATTN(true);
+  else MX_WATTN(false);
+#undef MX_WATTN
   return (int)hipGetLastError();
 }
 
