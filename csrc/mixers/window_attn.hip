@@ -93,7 +93,7 @@ __global__ void attn_prep_kernel(float* __restrict__ q_out, const T* __restrict_
 //  * otherwise lane = value column, one key at a time.
 // ---------------------------------------------------------------------------------
 constexpr int kWaves = 4;
-constexpr int kMaxVCols = 4;          // value columns per lane (scalar form): dv <= 256
+constexpr int kMaxVCols = 8;          // value columns per lane (scalar form): dv <= 512
 
 template <typename TC> struct Piece;
 template <> struct Piece<float> {

@@ -183,6 +183,11 @@ def save_checkpoint(cfg: BagasunConfig, tensors: Dict[str, torch.Tensor], out_di
         json.dump(config_to_dict(cfg), f, indent=1)
 
 
+def _window(mixer: dict) -> int:
+    """Keys a position sees, itself included (0: every earlier key, when no mask is given)."""
+    return int((mixer.get("mask") or {}).get("size", 0))
+
+
 class BagasunModel(StackedModel):
     family = "Bagasun"
 
@@ -203,13 +208,13 @@ class BagasunModel(StackedModel):
                                         m["conv"], m.get("norm_groups", 1), eps, dt, dev)
             elif l["type"] == SIGMOID:
                 mixer = SigmoidAttention(mget, width, m["heads"], m.get("kv_heads", m["heads"]), m["dim"],
-                                         m["vdim"], m["mask"]["size"], m["scale"], eps, dt, dev)
+                                         m["vdim"], _window(m), m["scale"], eps, dt, dev)
             else:
                 rot = m.get("rot") or {}
                 sc = rot.get("scaling")
                 mixer = DifferentialAttention(
                     mget, width, m["heads"], m.get("kv_heads", m["heads"]), m["dim"], m["vdim"],
-                    m["mask"]["size"], m["scale"], m["diff"], int(rot.get("dims", 0)),
+                    _window(m), m["scale"], m["diff"], int(rot.get("dims", 0)),
                     float(rot.get("base", 10000.0)),
                     (sc["factor"], sc["low"], sc["high"], sc["original"]) if sc else None, eps, dt, dev, max_pos)
             nw = lambda n, p=p: self.norm_weight(get(p + n))   # noqa: E731

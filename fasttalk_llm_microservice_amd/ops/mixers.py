@@ -398,6 +398,10 @@ def window_attention_products(out, q, k_cache, v_cache, seg: Segments, spec: Win
         if n < min_rows:
             continue
         step = PRODUCT_CHUNK_ROWS if sp.window <= 0 else max(PRODUCT_CHUNK_ROWS, min(sp.window, 1024))
+        # the fp32 scores of a chunk ([heads*maps, rows, keys]) stay under PRODUCT_SCORE_BYTES
+        span = sp.window if sp.window > 0 else kv_len[s]
+        while step > 32 and 4 * sp.heads * sp.maps * step * (step + span) > PRODUCT_SCORE_BYTES:
+            step //= 2
         for c0 in range(0, n, step):
             c1 = min(n, c0 + step)
             rows = c1 - c0
