@@ -35,7 +35,7 @@ def test_attn_prep(dt, norm, rot):
     t = 15
     qkv = rnd(t, nq + nk + nv + 3, dt=dt, g=g)[:, :nq + nk + nv]       # rows wider than the op's part
     wq, wk = (1 + rnd(nq, g=g, scale=0.2), 1 + rnd(nk, g=g, scale=0.2)) if norm else (None, None)
-    table = M.rope_table(40, rot, 50.0, scaling=(4.0, 1.0, 4.0, 30)) if rot else None
+    table = M.rope_table(40, rot, 50.0, scaling=(3.0, 0.5, 2.0, 30)) if rot else None
     pos = torch.tensor([3, 4, 5, 6, 7, 20, 0, 1, 2, 3, 4, 5, 6, 7, 8], dtype=torch.int32)
     slots = torch.randperm(blocks * 4)[:t].int()
     slots[4] = -1                                                       # a padding row writes nothing
