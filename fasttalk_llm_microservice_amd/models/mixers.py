@@ -202,10 +202,11 @@ class WindowedAttention:
 
 
 class SigmoidAttention(WindowedAttention):
-    """Windowed attention without softmax: q, k, v projections with biases, an RMS norm
-    over the whole q projection and over the whole k projection (weights of that size),
-    no rotation; a key's weight is sigmoid(q.k * scale - r1_h ln(1 + r2_h (i - j)) + pb_h),
-    not normalised over keys."""
+    """Windowed attention whose weights are independent sigmoids instead of a softmax:
+    w_ij = sigmoid(q_i.k_j * scale - r1_h ln(1 + r2_h (i - j)) + pb_h) for every key in
+    the window, and the output is sum_j w_ij v_j as it stands.  q, k and v come from
+    biased projections; all rows of q together (and all rows of k together) pass one RMS
+    norm with a weight per row; positions enter through the distance term only."""
 
     def __init__(self, get: Get, width: int, heads: int, kv_heads: int, dim: int, vdim: int,
                  window: int, scale: float, eps: float, dtype, device):
@@ -228,12 +229,14 @@ class SigmoidAttention(WindowedAttention):
 
 
 class DifferentialAttention(WindowedAttention):
-    """Windowed differential attention: two softmax score maps per head ([map 1, map 2]
-    rows of q and k, head by head) over the same values, o = a1 - lam a2 with
-    lam = exp(lq1.lk1) - exp(lq2.lk2) + diff, o divided by its root mean square per head,
-    times (1 - diff), times a per-head sigmoid gate of the mixer's input.  Rotary
-    positions on the first ``rot_dims`` entries of every map (optionally with
-    wavelength-dependent frequency scaling)."""
+    """Windowed attention that subtracts a second softmax map from the first.  For each
+    head in turn, q and k hold the rows of its map-0 projection and then of its map-1
+    projection; both maps weight one shared set of values, giving a_0 and a_1.  Output
+    per head: o = a_0 - lam a_1 with the layer constant
+    lam = exp(<lq1, lk1>) - exp(<lq2, lk2>) + diff; then o / rms(o) * (1 - diff) *
+    sigmoid(g_h), where g = W_g x is one gate logit per head taken from the mixer's input.
+    The first ``rot_dims`` entries of every map's q and k rows are rotated by position
+    (frequencies optionally rescaled by wavelength, :func:`ops.mixers_ref.scale_frequencies`)."""
 
     def __init__(self, get: Get, width: int, heads: int, kv_heads: int, dim: int, vdim: int,
                  window: int, scale: float, diff: float, rot_dims: int, rot_base: float, rot_scaling,

@@ -39,9 +39,10 @@ def add_rms_norm_rows(residual, y, wb, eps, add_vec, next_w, out_dtype, want_cas
 
 
 def scale_frequencies(f, factor: float, low: float, high: float, original: float):
-    """Long-context rescaling of rotary frequencies by wavelength l = 2 pi / f: kept
-    where l < original / high, divided by ``factor`` where l > original / low, and
-    blended linearly in ``original / l`` between the two."""
+    """Rotary frequencies stretched for long contexts.  With t_i = original * f_i / (2 pi)
+    (how many turns pair i makes over ``original`` positions): f_i stays for t_i > high,
+    becomes f_i / factor for t_i < low, and for low <= t_i <= high is the mix
+    (1 - s) f_i / factor + s f_i with s = (t_i - low) / (high - low)."""
     wl = 2.0 * math.pi / f
     s = ((original / wl - low) / (high - low)).clamp(0.0, 1.0)
     mid = (1.0 - s) * f / factor + s * f
