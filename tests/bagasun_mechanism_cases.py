@@ -1,8 +1,6 @@
 """Each Bagasun mechanism of models/mixers.py (and the ops under it) alone against the
 oracle's function for it: one whole sequence, then the same sequence cut in two steps
 through the cache / state the first step left; with and without the banded products."""
-import math
-
 import torch
 
 import bagasun_oracle as O
